@@ -1,0 +1,142 @@
+/*
+ * svdq_amd.h -- C ABI of the MI355X (gfx950) SVDQuant W4A4 + low-rank linear path.
+ *
+ * This is the drop-in boundary for the two operators that nunchaku exposes from its native
+ * module as `_C.ops.quantize_w4a4_act_fuse_lora` and `_C.ops.gemm_w4a4`
+ * (reference: nunchaku/csrc/pybind.cpp:108-110, nunchaku/csrc/ops.h:10-110), plus the one-time
+ * load-time conversion of reference-format checkpoint tensors into the layouts these kernels read.
+ *
+ * Conventions
+ *   - plain pointers to DEVICE memory, sizes as int64_t, no framework types;
+ *   - every function only enqueues work on `stream` (a hipStream_t passed as void*) and returns;
+ *     no allocation, no synchronisation, no global state: safe to call from several threads;
+ *   - return value 0 on success, a negative SVDQ_E* code otherwise; arguments are validated before
+ *     anything is launched, so a failed call has no side effect;
+ *   - `svdq_last_error()` returns a thread-local human-readable message for the last failure.
+ *
+ * Notation: M tokens, M_pad = M rounded up to 256, K in-features, N out-features, R low-rank rank,
+ * G group size (64 for INT4, 16 for NVFP4).
+ */
+#ifndef SVDQ_AMD_H
+#define SVDQ_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SVDQ_OK 0
+#define SVDQ_EINVAL -1       /* null pointer, bad shape, bad alignment */
+#define SVDQ_EUNSUPPORTED -2 /* valid request that this build does not implement */
+#define SVDQ_ELAUNCH -3      /* the HIP runtime refused the launch */
+
+#define SVDQ_ABI_VERSION 1
+
+int svdq_abi_version(void);
+const char *svdq_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Load-time repack: reference storage layout -> native layout.  Each runs once per tensor.
+ * The reference layouts are the ones NunchakuWeightPacker writes
+ * (nunchaku/lora/flux/packer.py:187-398) and the CUDA loaders read
+ * (src/kernels/zgemm/gemm_base.cuh:265-340,474-489, lora.cuh:43-59, gemm_w4a4.cuh:46-83).
+ * ------------------------------------------------------------------------------------------ */
+
+/* qweight int8 [N, K/2] (reference lane order, two's complement nibbles)
+ *   -> native int8 [N, K/2]: tiles [N/32][K/64][32 rows][32 bytes], byte b of a (row, group) holds
+ *      elements 2b (low nibble) and 2b+1 (high nibble).  INT4 codes are stored offset-binary
+ *      (code + 8); NVFP4 patterns (fp4 != 0) are stored unchanged.
+ * Replaces the implicit layout contract of packed_wgt_t loads, gemm_base.cuh:278-294. */
+int svdq_repack_qweight(const void *src, void *dst, int64_t N, int64_t K, int fp4, void *stream);
+
+/* wscales bf16 [K/64, N] (reference lane order) -> native:
+ *   dst_scales fp16 [K/64, N]  = wscales[g, n] * 2^e[n]   (column-normalised so that the largest
+ *                               scale of a column lies in [2^11, 2^12); exact, power-of-two shift)
+ *   dst_colnorm fp32 [N]       = 2^-e[n]
+ * Replaces packed_wscale_t loads, gemm_base.cuh:474-489. */
+int svdq_repack_wscales(const void *src, void *dst_scales, void *dst_colnorm, int64_t N, int64_t K, void *stream);
+
+/* NVFP4 micro scales fp8-e4m3 [K/16, N] (reference lane order) -> native fp16 [K/16, N] and fp32
+ * colnorm [N], normalised as above.  Replaces packed_wmscale_t loads, gemm_w4a4.cuh:75-83. */
+int svdq_repack_wmscales(const void *src, void *dst_scales, void *dst_colnorm, int64_t N, int64_t K, void *stream);
+
+/* bias / smooth_factor / wcscales bf16 [N] (reference lane order) -> bf16 [N] in channel order.
+ * Replaces the packed_wscale_t view of these vectors, gemm_w4a4_launch_impl.cuh:186-187,294. */
+int svdq_repack_vector(const void *src, void *dst, int64_t N, void *stream);
+
+/* smooth_factor bf16 [K] (reference lane order) -> fp32 [K] holding the correctly rounded
+ * reciprocal 1/smooth[k] in channel order (what the quantizer multiplies by). */
+int svdq_repack_smooth(const void *src, void *dst_rcp, int64_t K, void *stream);
+
+/* proj_down bf16 [K, R] (reference lane order) -> native bf16 [K/128][4][R/16][64][8]: operand
+ * order of the 16x16x32 bf16 MFMA used by the quantize kernel.  Replaces lora.cuh:43-59. */
+int svdq_repack_lora_down(const void *src, void *dst, int64_t K, int64_t R, void *stream);
+
+/* proj_up bf16 [N, R] (reference lane order) -> bf16 [N, R] row-major in channel/rank order. */
+int svdq_repack_lora_up(const void *src, void *dst, int64_t N, int64_t R, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Operator 1: smooth + quantize activations + low-rank down projection, one pass over x.
+ * Replaces ops.quantize_w4a4_act_fuse_lora (nunchaku/csrc/ops.h:82-110 ->
+ * src/kernels/zgemm/gemm_w4a4_launch_impl.cuh:450-521, kernel gemm_w4a4.cuh:1097-1184).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct svdq_quantize_args {
+    const void *input;      /* bf16 [M, K] row-major */
+    void *output;           /* u8 [M_pad, K/2] native activation tiles [M_pad/32][K/G64][32][32 B];
+                               INT4 codes offset-binary (code + 8), NVFP4 patterns unchanged      */
+    void *oscales;          /* INT4: bf16 [K/64, M_pad]; NVFP4: fp8-e4m3 [K/16, M_pad]; group-major */
+    const void *lora_down;  /* native proj_down (svdq_repack_lora_down) or NULL when R == 0       */
+    float *lora_act_out;    /* fp32 [M_pad, R] row-major; fully written (no pre-zero needed)       */
+    const float *smooth_rcp;/* fp32 [K] from svdq_repack_smooth, or NULL for no smoothing          */
+    int64_t M, M_pad, K, R;
+    int32_t fp4;            /* 0: INT4 group 64 (signed); 1: NVFP4 group 16                        */
+    int32_t fuse_glu;       /* must be 0 (not implemented)                                         */
+} svdq_quantize_args;
+
+int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Operator 2: W4A4 GEMM with fused epilogue.
+ * Replaces ops.gemm_w4a4 (nunchaku/csrc/ops.h:10-80 -> gemm_w4a4_launch_impl.cuh:7-424, kernels
+ * gemm_w4a4.cuh:1046-1095 and :358-405).  Epilogue order (launch_impl.cuh:172-280):
+ *   acc * alpha * wcscales + bias -> + low-rank up -> GELU/SiLU -> [low-rank down of the next
+ *   layer] -> store bf16 `out` and/or shift + smooth + quantize for the next layer (`qout`).
+ * The GELU is applied exactly when `qout` is given (launch_impl.cuh:282-309).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct svdq_gemm_args {
+    const void *act;        /* u8 native activation tiles [M_pad, K/2]                              */
+    const void *ascales;    /* bf16 [K/64, M_pad] (INT4) or fp8-e4m3 [K/16, M_pad] (NVFP4)          */
+    const void *wgt;        /* native qweight (svdq_repack_qweight)                                 */
+    const void *wscales;    /* native fp16 scales (svdq_repack_wscales / _wmscales)                 */
+    const float *colnorm;   /* fp32 [N] from the same repack call                                   */
+    const void *bias;       /* bf16 [N] channel order, or NULL                                      */
+    const void *wcscales;   /* bf16 [N] channel order, or NULL                                      */
+    const float *lora_act_in; /* fp32 [M_pad, R_up] row-major, or NULL                              */
+    const void *lora_up;    /* bf16 [N, R_up] (svdq_repack_lora_up), or NULL                        */
+    const float *lora_scales; /* HOST pointer, ceil(R_up/16) floats, or NULL for all ones           */
+    void *out;              /* bf16 [M_out, N_out] row-major, or NULL                               */
+    /* next-layer fusion (all NULL unless qout is given) */
+    void *qout;             /* u8 native activation tiles [M_pad, N/2] for the next layer           */
+    void *oscales;          /* bf16 [N/64, M_pad] (INT4 unsigned) or fp8 [N/16, M_pad] (NVFP4)      */
+    const float *next_smooth_rcp; /* fp32 [N] from svdq_repack_smooth of the next layer             */
+    const void *next_lora_down;   /* native proj_down of the next layer ([N, R_down]) or NULL       */
+    float *next_lora_act_out;     /* fp32 [M_pad, R_down]; zeroed and accumulated by the call       */
+    int64_t M_pad, N, K;
+    int64_t M_out, N_out;   /* shape of `out` (M_out <= M_pad, N_out <= N)                          */
+    int64_t R_up, R_down;
+    float alpha;            /* per-tensor scale (NVFP4 wtscale); must be 1 for INT4                 */
+    int32_t act_unsigned;   /* INT4 activations are unsigned codes 0..15                            */
+    int32_t fuse_silu;      /* must be 0 (not implemented)                                          */
+    int32_t fp4;            /* operands are NVFP4                                                   */
+} svdq_gemm_args;
+
+int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
+
+
+
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SVDQ_AMD_H */

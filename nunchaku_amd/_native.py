@@ -1,0 +1,138 @@
+"""ctypes binding of ``libsvdq_amd.so`` (the C ABI declared in ``include/svdq_amd.h``) and the
+tensor-level helpers built on it.
+
+PyTorch is only used for device memory and streams: every call passes raw device pointers, sizes
+and the current HIP stream.  There is no fallback path: if the library is missing, or a tensor is
+not on a GPU, the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from pathlib import Path
+
+import torch
+
+_PKG_DIR = Path(__file__).resolve().parent
+_CSRC = _PKG_DIR / "csrc"
+LIB_PATH = _PKG_DIR / "libsvdq_amd.so"
+SOURCES = ["repack.hip", "quantize.hip", "gemm.hip"]
+HIPCC_FLAGS = [
+    "-shared", "-fPIC", "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+SVDQ_ABI_VERSION = 1
+EXPORTED_SYMBOLS = [
+    "svdq_abi_version", "svdq_last_error",
+    "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
+    "svdq_repack_smooth", "svdq_repack_lora_down", "svdq_repack_lora_up",
+    "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4",
+]
+
+
+class QuantizeArgs(ctypes.Structure):
+    """Mirror of ``svdq_quantize_args``."""
+
+    _fields_ = [
+        ("input", ctypes.c_void_p), ("output", ctypes.c_void_p), ("oscales", ctypes.c_void_p),
+        ("lora_down", ctypes.c_void_p), ("lora_act_out", ctypes.c_void_p), ("smooth_rcp", ctypes.c_void_p),
+        ("M", ctypes.c_int64), ("M_pad", ctypes.c_int64), ("K", ctypes.c_int64), ("R", ctypes.c_int64),
+        ("fp4", ctypes.c_int32), ("fuse_glu", ctypes.c_int32),
+    ]
+
+
+class GemmArgs(ctypes.Structure):
+    """Mirror of ``svdq_gemm_args``."""
+
+    _fields_ = [
+        ("act", ctypes.c_void_p), ("ascales", ctypes.c_void_p), ("wgt", ctypes.c_void_p),
+        ("wscales", ctypes.c_void_p), ("colnorm", ctypes.c_void_p), ("bias", ctypes.c_void_p),
+        ("wcscales", ctypes.c_void_p), ("lora_act_in", ctypes.c_void_p), ("lora_up", ctypes.c_void_p),
+        ("lora_scales", ctypes.POINTER(ctypes.c_float)), ("out", ctypes.c_void_p),
+        ("qout", ctypes.c_void_p), ("oscales", ctypes.c_void_p), ("next_smooth_rcp", ctypes.c_void_p),
+        ("next_lora_down", ctypes.c_void_p), ("next_lora_act_out", ctypes.c_void_p),
+        ("M_pad", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
+        ("M_out", ctypes.c_int64), ("N_out", ctypes.c_int64),
+        ("R_up", ctypes.c_int64), ("R_down", ctypes.c_int64),
+        ("alpha", ctypes.c_float), ("act_unsigned", ctypes.c_int32), ("fuse_silu", ctypes.c_int32),
+        ("fp4", ctypes.c_int32),
+    ]
+
+
+def build(verbose: bool = False) -> Path:
+    """Compile the HIP sources for gfx950 into ``libsvdq_amd.so`` next to this file (hipcc
+    cross-compiles; no GPU is needed)."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, *[str(_CSRC / s) for s in SOURCES], "-o", str(LIB_PATH)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stderr[-4000:])
+    if verbose:
+        print(" ".join(cmd))
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library.  Raises if it has not been built: there is no other implementation."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(the HIP extension is the only implementation of this path)"
+            )
+        L = ctypes.CDLL(str(LIB_PATH))
+        L.svdq_abi_version.restype = ctypes.c_int
+        L.svdq_last_error.restype = ctypes.c_char_p
+        i64, vp, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+        L.svdq_repack_qweight.argtypes = [vp, vp, i64, i64, ci, vp]
+        L.svdq_repack_wscales.argtypes = [vp, vp, vp, i64, i64, vp]
+        L.svdq_repack_wmscales.argtypes = [vp, vp, vp, i64, i64, vp]
+        L.svdq_repack_vector.argtypes = [vp, vp, i64, vp]
+        L.svdq_repack_smooth.argtypes = [vp, vp, i64, vp]
+        L.svdq_repack_lora_down.argtypes = [vp, vp, i64, i64, vp]
+        L.svdq_repack_lora_up.argtypes = [vp, vp, i64, i64, vp]
+        L.svdq_quantize_w4a4_act_fuse_lora.argtypes = [ctypes.POINTER(QuantizeArgs), vp]
+        L.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        for name in EXPORTED_SYMBOLS:
+            getattr(L, name)
+            if name not in ("svdq_last_error",):
+                getattr(L, name).restype = ctypes.c_int if name != "svdq_last_error" else ctypes.c_char_p
+        L.svdq_last_error.restype = ctypes.c_char_p
+        if L.svdq_abi_version() != SVDQ_ABI_VERSION:
+            raise RuntimeError("libsvdq_amd.so was built from a different header version; rebuild it")
+        _lib = L
+    return _lib
+
+
+def check(rc: int) -> None:
+    """Turn a C-ABI return code into the exception the reference's users expect."""
+    if rc == 0:
+        return
+    msg = lib().svdq_last_error().decode()
+    if rc == -1:
+        raise ValueError(msg)
+    if rc == -2:
+        raise NotImplementedError(msg)
+    raise RuntimeError(msg)
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on a GPU (got {t.device}); this path has no CPU implementation")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")

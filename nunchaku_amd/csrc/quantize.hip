@@ -1,0 +1,270 @@
+// Operator 1: activation smoothing + 4-bit quantization + low-rank down projection in one pass
+// over x.  Counterpart of quantize_w4a4_fuse_lora_kernel (src/kernels/zgemm/gemm_w4a4.cuh:1097-1184).
+//
+// Work split: one workgroup (4 waves) owns 16*MT consecutive rows for the whole K extent, so the
+// low-rank projection needs no atomics and no pre-zeroed output.  Wave w walks the 128-column
+// chunks c = w, w+4, ...  Inside a chunk lane (r = lane%16, q = lane/16) holds, for each 16-row
+// tile, the 32 consecutive columns 128c + 32q + [0, 32) of row r: half of a 64-group (INT4) or two
+// whole 16-groups (NVFP4).  The same registers feed the bf16 MFMA of the low-rank projection
+// (operand slot (q, j) of step i = column 128c + 32q + 8i + j; proj_down is stored in that order).
+//
+// Arithmetic (bit-exact contract; IEEE, round-to-nearest-even):
+//   y    = bf16(x / smooth)        computed as bf16(x * fl32(1/smooth)).  For bf16 operands this
+//                                  equals bf16(fl32(x / smooth)) bit for bit: the quotient of two
+//                                  8-bit significands is never a bf16 rounding midpoint and is
+//                                  otherwise at least 2^-16 (relative) away from one, while the two
+//                                  fp32 roundings of the product move it by less than 2^-22.
+//   amax = max |y| over the group; s = f32(amax) * fl32(1/7); stored scale bf16(s); r = fl32(1/s)
+//   code = clamp(rne(y * r), -8, 7)               (gemm_w4a4.cuh:429-523)
+//   NVFP4: s = min(f32(amax) * fl32(1/6), 448), stored e4m3(s), code = e2m1(y * fl32(1/s))
+//                                                  (gemm_w4a4.cuh:85-187)
+#include "svdq_common.h"
+
+using namespace svdq;
+
+namespace {
+
+constexpr float RECIP_7 = 1.0f / 7.0f;
+constexpr float RECIP_15 = 1.0f / 15.0f;
+constexpr float RECIP_6 = 1.0f / 6.0f;
+constexpr float RNE_MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds to an integer (RNE)
+
+__device__ inline float smooth_quotient(float x, float rcp) {
+    // bf16(x / smooth) as fp32, see the header comment
+    return bf16_bits_to_f32(f32_to_bf16_bits(__fmul_rn(x, rcp)));
+}
+
+// 8 clamped-and-rounded codes (already offset so that they are in [0, 15]) -> one word
+__device__ inline uint32_t pack8(const float (&v)[8]) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) w |= (f32_bits(v[j]) & 15u) << (4 * j);
+    return w;
+}
+
+// fp32 (finite, >= 0, <= 448) -> e4m3 bit pattern, round to nearest even
+__device__ inline uint32_t f32_to_e4m3(float s) {
+    if (s < 0.0009765625f) return 0;  // below half of the smallest subnormal (2^-10) rounds to 0
+    if (s < 0.015625f) {              // subnormal range: multiples of 2^-9
+        float t = __fadd_rn(__fmul_rn(s, 512.0f), RNE_MAGIC);
+        return f32_bits(t) & 0xFF;    // 0..8 (8 == smallest normal, pattern 0x08)
+    }
+    uint32_t b = f32_bits(s);
+    b += 0x7FFFFu + ((b >> 20) & 1u);  // round mantissa to 3 bits, ties to even
+    const int ex = (int)(b >> 23) - 127 + 7;
+    return (uint32_t)(ex << 3) | ((b >> 20) & 7u);
+}
+
+// fp32 -> 4-bit e2m1 pattern, round to nearest even, saturating at 6
+__device__ inline uint32_t f32_to_e2m1(float v) {
+    const float a = fabsf(v);
+    uint32_t c;
+    // grid 0 .5 1 1.5 2 3 4 6 ; ties go to the pattern with an even low bit
+    if (a <= 0.25f) c = 0;
+    else if (a < 0.75f) c = 1;
+    else if (a <= 1.25f) c = 2;
+    else if (a < 1.75f) c = 3;
+    else if (a <= 2.5f) c = 4;
+    else if (a < 3.5f) c = 5;
+    else if (a <= 5.0f) c = 6;
+    else c = 7;
+    return c | ((f32_bits(v) >> 28) & 8u);
+}
+
+struct QuantParams {
+    const uint16_t *x;       // bf16 [M, K]
+    uint8_t *act;            // native tiles
+    void *oscales;           // bf16 [K/64, M_pad] or fp8 [K/16, M_pad]
+    const bf16x8_t *down;    // native proj_down
+    float *lora_out;         // [M_pad, R]
+    const float *smooth_rcp; // [K] or null
+    int M, M_pad, K, R;
+};
+
+template <int MT, int RT_MAX, bool FP4>
+__global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) {
+    extern __shared__ float red[];  // [4 waves][MT][RT][64][4]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int row0 = blockIdx.x * (16 * MT);
+    const int kgroups = p.K / 64;
+    const int RT = p.R / 16;
+
+    float4_t acc[MT][RT_MAX];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int rt = 0; rt < RT_MAX; rt++) acc[mt][rt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int c = wave; c < p.K / 128; c += 4) {
+        const int kbase = 128 * c + 32 * q;
+        // ---- load x: MT tiles x 4 steps x 8 bf16
+        u32x4_t xv[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            const int row = row0 + 16 * mt + r;
+            const u32x4_t *src = (const u32x4_t *)(p.x + (size_t)row * p.K + kbase);
+#pragma unroll
+            for (int i = 0; i < 4; i++) xv[mt][i] = row < p.M ? src[i] : u32x4_t{0, 0, 0, 0};
+        }
+        // ---- reciprocal smoothing factors of my 32 columns
+        float rs[32];
+        if (p.smooth_rcp) {
+            const float4_t *sp = (const float4_t *)(p.smooth_rcp + kbase);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float4_t v = sp[i];
+                rs[4 * i] = v[0]; rs[4 * i + 1] = v[1]; rs[4 * i + 2] = v[2]; rs[4 * i + 3] = v[3];
+            }
+        }
+        // ---- low-rank down projection on the raw activations
+        if (RT > 0) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+#pragma unroll
+                for (int rt = 0; rt < RT_MAX; rt++) {
+                    if (rt < RT) {
+                        const bf16x8_t b = p.down[((size_t)(c * 4 + i) * RT + rt) * 64 + lane];
+#pragma unroll
+                        for (int mt = 0; mt < MT; mt++) {
+                            bf16x8_t a = __builtin_bit_cast(bf16x8_t, xv[mt][i]);
+                            acc[mt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt][rt], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        // ---- smooth, quantize, store
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            const int row = row0 + 16 * mt + r;
+            float y[32];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t w = xv[mt][i][j];
+                    const float lo = bits_f32(w << 16), hi = bits_f32(w & 0xFFFF0000u);
+                    const int e = 8 * i + 2 * j;
+                    y[e] = p.smooth_rcp ? smooth_quotient(lo, rs[e]) : lo;
+                    y[e + 1] = p.smooth_rcp ? smooth_quotient(hi, rs[e + 1]) : hi;
+                }
+            }
+            const size_t tile = (size_t)(row / 32) * kgroups + (2 * c + (q >> 1));
+            uint8_t *dst = p.act + tile * TILE_BYTES + (row % 32) * 32 + 16 * (q & 1);
+            u32x4_t words;
+            if (!FP4) {
+                float amax = 0.f;
+#pragma unroll
+                for (int e = 0; e < 32; e++) amax = fmaxf(amax, fabsf(y[e]));
+                amax = fmaxf(amax, __shfl_xor(amax, 16));
+                const float s = __fmul_rn(amax, RECIP_7);
+                const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
+#pragma unroll
+                for (int wi = 0; wi < 4; wi++) {
+                    float v[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        float t = __fmul_rn(y[8 * wi + j], rcp);
+                        t = fminf(fmaxf(t, -8.0f), 7.0f);
+                        v[j] = __fadd_rn(t, RNE_MAGIC + 8.0f);  // offset-binary code in the low nibble
+                    }
+                    words[wi] = pack8(v);
+                }
+                if ((q & 1) == 0)
+                    ((uint16_t *)p.oscales)[(size_t)(2 * c + (q >> 1)) * p.M_pad + row] = (uint16_t)f32_to_bf16_bits(s);
+            } else {
+                uint32_t sc[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    float amax = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 16; e++) amax = fmaxf(amax, fabsf(y[16 * h + e]));
+                    const float s = fminf(__fmul_rn(amax, RECIP_6), 448.0f);
+                    const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
+                    sc[h] = f32_to_e4m3(s);
+#pragma unroll
+                    for (int wi = 0; wi < 2; wi++) {
+                        uint32_t w = 0;
+#pragma unroll
+                        for (int j = 0; j < 8; j++) w |= f32_to_e2m1(s > 0.f ? __fmul_rn(y[16 * h + 8 * wi + j], rcp) : 0.f) << (4 * j);
+                        words[2 * h + wi] = w;
+                    }
+                }
+                uint8_t *os = (uint8_t *)p.oscales;
+                os[(size_t)(8 * c + 2 * q) * p.M_pad + row] = (uint8_t)sc[0];
+                os[(size_t)(8 * c + 2 * q + 1) * p.M_pad + row] = (uint8_t)sc[1];
+            }
+            *(u32x4_t *)dst = words;
+        }
+    }
+
+    // ---- reduce the four waves' partial projections and write lora_act[row][rank]
+    if (RT > 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int rt = 0; rt < RT_MAX; rt++)
+                if (rt < RT) *(float4_t *)&red[(((wave * MT + mt) * RT + rt) * 64 + lane) * 4] = acc[mt][rt];
+        __syncthreads();
+        const int total = 16 * MT * p.R;
+        for (int idx = threadIdx.x; idx < total; idx += 256) {
+            const int row = idx / p.R, rank = idx % p.R;
+            const int mt = row / 16, rr = row % 16, rt = rank / 16, rc = rank % 16;
+            const int src_lane = 16 * (rr / 4) + rc, i = rr % 4;  // 16x16 MFMA result layout
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) sum += red[(((w * MT + mt) * RT + rt) * 64 + src_lane) * 4 + i];
+            p.lora_out[(size_t)(row0 + row) * p.R + rank] = sum;
+        }
+    }
+}
+
+template <int MT, int RT_MAX, bool FP4>
+int launch(const QuantParams &p, hipStream_t stream) {
+    const size_t smem = (size_t)4 * MT * (p.R / 16) * 64 * 4 * sizeof(float);
+    auto kern = quantize_fuse_lora_kernel<MT, RT_MAX, FP4>;
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "quantize: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3(p.M_pad / (16 * MT)), dim3(256), smem, stream, p);
+    return check_launch("quantize_w4a4_act_fuse_lora");
+}
+
+template <bool FP4>
+int dispatch(const QuantParams &p, hipStream_t stream) {
+    // rows per workgroup: enough workgroups to cover the chip, but amortise proj_down reads at high rank
+    const int RT = p.R / 16;
+    if (RT <= 2) return p.M_pad >= 8192 ? launch<2, 2, FP4>(p, stream) : launch<1, 2, FP4>(p, stream);
+    if (RT <= 4) return launch<2, 4, FP4>(p, stream);
+    if (RT <= 8) return launch<2, 8, FP4>(p, stream);
+    return fail(SVDQ_EUNSUPPORTED, "quantize: rank %d > 128 is not supported", p.R);
+}
+
+}  // namespace
+
+extern "C" int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *a, void *stream) {
+    SVDQ_REQUIRE(a, "quantize: null args");
+    SVDQ_REQUIRE(a->input && a->output && a->oscales, "quantize: input/output/oscales must not be null");
+    SVDQ_REQUIRE(a->M > 0 && a->M_pad >= a->M && a->M_pad % 256 == 0, "quantize: M_pad (%lld) must be a multiple of 256 and >= M (%lld)",
+                 (long long)a->M_pad, (long long)a->M);
+    SVDQ_REQUIRE(a->K > 0 && a->K % 128 == 0, "quantize: K (%lld) must be a multiple of 128", (long long)a->K);
+    SVDQ_REQUIRE(a->R >= 0 && a->R % 16 == 0, "quantize: rank (%lld) must be a multiple of 16", (long long)a->R);
+    SVDQ_REQUIRE(a->R == 0 || (a->lora_down && a->lora_act_out), "quantize: lora_down/lora_act_out must be given when R > 0");
+    SVDQ_REQUIRE(a->M_pad < (1ll << 31) / 4 && a->K < (1 << 24), "quantize: shape too large");
+    SVDQ_REQUIRE(((uintptr_t)a->input % 16 == 0) && ((uintptr_t)a->output % 16 == 0) && ((uintptr_t)a->lora_down % 16 == 0) &&
+                     ((uintptr_t)a->smooth_rcp % 16 == 0),
+                 "quantize: pointers must be 16-byte aligned");
+    if (a->fuse_glu) return fail(SVDQ_EUNSUPPORTED, "quantize: fuse_glu is not implemented");
+    QuantParams p;
+    p.x = (const uint16_t *)a->input;
+    p.act = (uint8_t *)a->output;
+    p.oscales = a->oscales;
+    p.down = (const bf16x8_t *)a->lora_down;
+    p.lora_out = a->lora_act_out;
+    p.smooth_rcp = a->smooth_rcp;
+    p.M = (int)a->M; p.M_pad = (int)a->M_pad; p.K = (int)a->K; p.R = (int)a->R;
+    return a->fp4 ? dispatch<true>(p, (hipStream_t)stream) : dispatch<false>(p, (hipStream_t)stream);
+}

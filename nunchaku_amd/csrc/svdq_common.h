@@ -1,0 +1,74 @@
+// Shared host/device helpers of the gfx950 SVDQuant W4A4 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/svdq_amd.h"
+
+namespace svdq {
+
+// ---- error reporting (thread local, no allocation) ---------------------------------------------
+inline char *err_buf() {
+    static thread_local char buf[512] = {0};
+    return buf;
+}
+inline int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(err_buf(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
+inline int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return SVDQ_OK;
+}
+#define SVDQ_REQUIRE(cond, ...) \
+    do {                        \
+        if (!(cond)) return svdq::fail(SVDQ_EINVAL, __VA_ARGS__); \
+    } while (0)
+
+// ---- vector types -------------------------------------------------------------------------------
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+// ---- bf16 <-> fp32 bit helpers ------------------------------------------------------------------
+__host__ __device__ inline float bf16_bits_to_f32(uint32_t b) {
+    union { uint32_t u; float f; } v;
+    v.u = b << 16;
+    return v.f;
+}
+__host__ __device__ inline uint32_t f32_bits(float f) {
+    union { uint32_t u; float f; } v;
+    v.f = f;
+    return v.u;
+}
+__host__ __device__ inline float bits_f32(uint32_t u) {
+    union { uint32_t u; float f; } v;
+    v.u = u;
+    return v.f;
+}
+// round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs)
+__host__ __device__ inline uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = f32_bits(f);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+// Native tile geometry of 4-bit operands (activations and weights alike):
+//   [rows/32][K/64][32 rows][32 bytes], byte b of a (row, 64-group) = elements 2b | (2b+1) << 4.
+constexpr int TILE_ROWS = 32;
+constexpr int GROUP_K = 64;
+constexpr int TILE_BYTES = TILE_ROWS * GROUP_K / 2;  // 1024
+
+}  // namespace svdq

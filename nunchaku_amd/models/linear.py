@@ -1,0 +1,154 @@
+"""``SVDQW4A4Linear`` with the constructor, parameter names/shapes/dtypes and methods of
+nunchaku/models/linear.py:9-135, so that a reference checkpoint's state dict loads unchanged.
+
+The parameters keep the reference storage layout (that is what checkpoints hold).  The first use
+after loading converts them once into the gfx950-native layouts (``native_tensors``); the converted
+tensors are what the kernels read.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .. import packing
+from ..ops.gemm import svdq_gemm_w4a4
+from ..ops.quantize import svdq_quantize_w4a4_act_fuse_lora
+
+
+class SVDQW4A4Linear(nn.Module):
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        rank: int = 32,
+        bias: bool = True,
+        precision: str = "int4",
+        act_unsigned: bool = False,
+        torch_dtype: torch.dtype = torch.bfloat16,
+        device: str | torch.device | None = None,
+    ):
+        super().__init__()
+        if device is None:
+            device = torch.device("cpu")
+        self.in_features = in_features
+        self.out_features = out_features
+        self.rank = rank
+        self.precision = precision
+        self.torch_dtype = torch_dtype
+        if precision == "nvfp4":
+            self.group_size = 16
+        elif precision == "int4":
+            self.group_size = 64
+        else:
+            raise ValueError(f"Invalid precision: {precision}")
+        if torch_dtype != torch.bfloat16:
+            raise NotImplementedError("only torch.bfloat16 layers are supported")
+
+        self.qweight = nn.Parameter(torch.empty(out_features, in_features // 2, dtype=torch.int8, device=device), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(out_features, dtype=torch_dtype, device=device), requires_grad=True) if bias else None
+        self.wscales = nn.Parameter(
+            torch.empty(
+                in_features // self.group_size, out_features,
+                dtype=torch_dtype if precision == "int4" else torch.float8_e4m3fn, device=device,
+            ),
+            requires_grad=False,
+        )
+        self.smooth_factor = nn.Parameter(torch.empty(in_features, dtype=torch_dtype, device=device), requires_grad=False)
+        self.smooth_factor_orig = nn.Parameter(torch.empty(in_features, dtype=torch_dtype, device=device), requires_grad=False)
+        self.proj_down = nn.Parameter(torch.empty(in_features, rank, dtype=torch_dtype, device=device))
+        self.proj_up = nn.Parameter(torch.empty(out_features, rank, dtype=torch_dtype, device=device))
+
+        self.wtscale = None
+        self.wcscales = None
+        if precision == "nvfp4":
+            self.wtscale = nn.Parameter(torch.ones(1, dtype=torch_dtype, device=device), requires_grad=False)
+            self.wcscales = nn.Parameter(torch.ones(out_features, dtype=torch_dtype, device=device), requires_grad=False)
+
+        self.act_unsigned = act_unsigned
+        self._native: dict[str, torch.Tensor | None] | None = None
+        self._alpha: float | None = None
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, **kwargs):
+        in_features = kwargs.pop("in_features", linear.in_features)
+        return cls(
+            in_features=in_features,
+            out_features=linear.out_features,
+            bias=linear.bias is not None,
+            torch_dtype=linear.weight.dtype,
+            device=linear.weight.device,
+            **kwargs,
+        )
+
+    # ---- load-time repack -------------------------------------------------------------------
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._native = None  # new checkpoint tensors: convert again on next use
+        self._alpha = None
+        return super()._load_from_state_dict(*args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        self._native = None
+        return super()._apply(fn, *args, **kwargs)
+
+    def native_tensors(self) -> dict[str, torch.Tensor | None]:
+        """The layer's tensors in the layouts the kernels read, converted on first use."""
+        if self._native is None:
+            fp4 = self.precision == "nvfp4"
+            self._native = {
+                "qweight": packing.repack_qweight(self.qweight.data, fp4),
+                "wscales": packing.repack_wscales(self.wscales.data, fp4),
+                "smooth_factor": packing.repack_smooth(self.smooth_factor.data),
+                "proj_down": packing.repack_lora_down(self.proj_down.data),
+                "proj_up": packing.repack_lora_up(self.proj_up.data),
+                "bias": None if self.bias is None else packing.repack_vector(self.bias.data),
+                "wcscales": None if self.wcscales is None else packing.repack_vector(self.wcscales.data),
+            }
+        return self._native
+
+    @property
+    def alpha(self) -> float:
+        """Per-tensor weight scale as a host float, read once (the reference hands the parameter to a
+        ``float`` argument on every call, nunchaku/models/linear.py:128, which synchronises)."""
+        if self._alpha is None:
+            self._alpha = 1.0 if self.wtscale is None else float(self.wtscale.detach().float().cpu().item())
+        return self._alpha
+
+    # ---- forward path (nunchaku/models/linear.py:89-132) ----------------------------------------
+    def forward(self, x: torch.Tensor, output: torch.Tensor | None = None) -> torch.Tensor:
+        batch_size, seq_len, channels = x.shape
+        x = x.view(batch_size * seq_len, channels)
+        if output is None:
+            output = torch.empty(batch_size * seq_len, self.out_features, dtype=x.dtype, device=x.device)
+        quantized_x, ascales, lora_act_out = self.quantize(x)
+        output = self.forward_quant(quantized_x, ascales, lora_act_out, output)
+        return output.view(batch_size, seq_len, -1)
+
+    def quantize(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        t = self.native_tensors()
+        return svdq_quantize_w4a4_act_fuse_lora(
+            x, lora_down=t["proj_down"], smooth=t["smooth_factor"], fp4=self.precision == "nvfp4"
+        )
+
+    def forward_quant(
+        self,
+        quantized_x: torch.Tensor,
+        ascales: torch.Tensor,
+        lora_act: torch.Tensor,
+        output: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        if output is None:
+            output = torch.empty(quantized_x.shape[0], self.out_features, dtype=self.proj_up.dtype, device=quantized_x.device)
+        t = self.native_tensors()
+        svdq_gemm_w4a4(
+            act=quantized_x, wgt=t["qweight"], out=output, ascales=ascales, wscales=t["wscales"],
+            lora_act_in=lora_act, lora_up=t["proj_up"], bias=t["bias"], fp4=self.precision == "nvfp4",
+            alpha=self.alpha, wcscales=t["wcscales"], act_unsigned=self.act_unsigned,
+        )
+        return output
+
+    def __repr__(self):
+        return (
+            f"SVDQW4A4Linear(in_features={self.in_features}, out_features={self.out_features}, rank={self.rank}, "
+            f"precision={self.precision}, act_unsigned={self.act_unsigned})"
+        )

@@ -1,0 +1,13 @@
+"""Operator wrappers with the signatures of ``nunchaku.ops`` (nunchaku/ops/{quantize,gemm,fused}.py)."""
+
+from .fused import fused_gelu_mlp
+from .gemm import svdq_gemm_w4a4, svdq_gemm_w4a4_cuda
+from .quantize import svdq_quantize_w4a4_act_fuse_lora, svdq_quantize_w4a4_act_fuse_lora_cuda
+
+__all__ = [
+    "svdq_quantize_w4a4_act_fuse_lora",
+    "svdq_quantize_w4a4_act_fuse_lora_cuda",
+    "svdq_gemm_w4a4",
+    "svdq_gemm_w4a4_cuda",
+    "fused_gelu_mlp",
+]

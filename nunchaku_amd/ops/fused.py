@@ -1,0 +1,35 @@
+"""``fused_gelu_mlp`` with the signature of nunchaku/ops/fused.py:10-47."""
+
+from __future__ import annotations
+
+import torch
+
+from ..utils import ceil_divide
+from .gemm import svdq_gemm_w4a4
+
+
+def fused_gelu_mlp(x: torch.Tensor, fc1, fc2, pad_size: int = 256) -> torch.Tensor:
+    """fc1 -> GELU -> fc2 with the GELU, fc2's activation quantization (unsigned INT4 after a
+    +0.171875 shift) and fc2's low-rank down projection fused into fc1's GEMM epilogue."""
+    batch_size, seq_len, channels = x.shape
+    x = x.view(batch_size * seq_len, channels)
+    quantized_x, ascales, lora_act = fc1.quantize(x)
+
+    batch_size_pad = ceil_divide(batch_size * seq_len, pad_size) * pad_size
+    qout_act = torch.empty(batch_size_pad, fc1.out_features // 2, dtype=torch.uint8, device=x.device)
+    if fc2.precision == "nvfp4":
+        qout_ascales = torch.empty(fc1.out_features // 16, batch_size_pad, dtype=torch.float8_e4m3fn, device=x.device)
+    else:
+        qout_ascales = torch.empty(fc1.out_features // 64, batch_size_pad, dtype=x.dtype, device=x.device)
+    qout_lora_act = torch.empty(batch_size_pad, fc2.proj_down.shape[1], dtype=torch.float32, device=x.device)
+
+    t1, t2 = fc1.native_tensors(), fc2.native_tensors()
+    svdq_gemm_w4a4(
+        act=quantized_x, wgt=t1["qweight"], qout=qout_act, ascales=ascales, wscales=t1["wscales"],
+        oscales=qout_ascales, lora_act_in=lora_act, lora_up=t1["proj_up"], lora_down=t2["proj_down"],
+        lora_act_out=qout_lora_act, bias=t1["bias"], smooth_factor=t2["smooth_factor"],
+        fp4=fc1.precision == "nvfp4", alpha=fc1.alpha, wcscales=t1["wcscales"],
+    )
+    output = torch.empty(batch_size * seq_len, fc2.out_features, dtype=x.dtype, device=x.device)
+    output = fc2.forward_quant(qout_act, qout_ascales, qout_lora_act, output=output)
+    return output.view(batch_size, seq_len, -1)

@@ -1,0 +1,146 @@
+"""Load-time repack of reference-format checkpoint tensors into the gfx950-native layouts, and the
+inverse views the tests need to compare kernel outputs in logical order.
+
+Reference formats: ``NunchakuWeightPacker`` (nunchaku/lora/flux/packer.py:187-398).  The byte
+shuffling itself runs on the GPU behind the C ABI (``svdq_repack_*``); this module only allocates
+the destination tensors and keeps a small cache so that an operator called with a reference-format
+tensor (as nunchaku.ops callers do) repacks it once, not per call.
+"""
+
+from __future__ import annotations
+
+import weakref
+
+import torch
+
+from . import _native as nv
+
+NATIVE_ATTR = "_svdq_native"
+
+
+def _tag(t: torch.Tensor, kind: str, **extra) -> torch.Tensor:
+    setattr(t, NATIVE_ATTR, kind)
+    for k, v in extra.items():
+        setattr(t, k, v)
+    return t
+
+
+def is_native(t: torch.Tensor | None, kind: str) -> bool:
+    return t is not None and getattr(t, NATIVE_ATTR, None) == kind
+
+
+def repack_qweight(qweight: torch.Tensor, fp4: bool = False) -> torch.Tensor:
+    """int8 [N, K/2] reference order -> int8 [N, K/2] native tiles (offset-binary INT4 codes)."""
+    nv.require_gpu(qweight, "qweight")
+    N, K2 = qweight.shape
+    out = torch.empty_like(qweight)
+    nv.check(nv.lib().svdq_repack_qweight(qweight.data_ptr(), out.data_ptr(), N, K2 * 2, int(fp4), nv.stream_ptr(qweight.device)))
+    return _tag(out, "qweight")
+
+
+def repack_wscales(wscales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
+    """bf16 [K/64, N] (or fp8 [K/16, N]) reference order -> fp16 column-normalised scales of the same
+    shape; the fp32 per-column factor that undoes the normalisation rides along as ``.colnorm``."""
+    nv.require_gpu(wscales, "wscales")
+    G, N = wscales.shape
+    out = torch.empty(G, N, dtype=torch.float16, device=wscales.device)
+    colnorm = torch.empty(N, dtype=torch.float32, device=wscales.device)
+    fn = nv.lib().svdq_repack_wmscales if fp4 else nv.lib().svdq_repack_wscales
+    K = G * (16 if fp4 else 64)
+    nv.check(fn(wscales.data_ptr(), out.data_ptr(), colnorm.data_ptr(), N, K, nv.stream_ptr(wscales.device)))
+    return _tag(out, "wscales", colnorm=colnorm)
+
+
+def repack_vector(vec: torch.Tensor) -> torch.Tensor:
+    """bias / wcscales / smooth_factor bf16 [N]: reference lane order -> channel order."""
+    nv.require_gpu(vec, "vector")
+    out = torch.empty_like(vec)
+    nv.check(nv.lib().svdq_repack_vector(vec.data_ptr(), out.data_ptr(), vec.numel(), nv.stream_ptr(vec.device)))
+    return _tag(out, "vector")
+
+
+def repack_smooth(smooth: torch.Tensor) -> torch.Tensor:
+    """smooth_factor bf16 [K] reference lane order -> fp32 [K] correctly rounded reciprocals."""
+    nv.require_gpu(smooth, "smooth_factor")
+    out = torch.empty(smooth.numel(), dtype=torch.float32, device=smooth.device)
+    nv.check(nv.lib().svdq_repack_smooth(smooth.data_ptr(), out.data_ptr(), smooth.numel(), nv.stream_ptr(smooth.device)))
+    return _tag(out, "smooth_rcp")
+
+
+def repack_lora_down(proj_down: torch.Tensor) -> torch.Tensor:
+    """bf16 [K, R] reference order -> native MFMA operand order (same shape and dtype)."""
+    nv.require_gpu(proj_down, "proj_down")
+    K, R = proj_down.shape
+    out = torch.empty_like(proj_down)
+    if R == 0:  # a layer without a low-rank branch
+        return _tag(out, "lora_down")
+    nv.check(nv.lib().svdq_repack_lora_down(proj_down.data_ptr(), out.data_ptr(), K, R, nv.stream_ptr(proj_down.device)))
+    return _tag(out, "lora_down")
+
+
+def repack_lora_up(proj_up: torch.Tensor) -> torch.Tensor:
+    """bf16 [N, R] reference order -> row-major channel/rank order."""
+    nv.require_gpu(proj_up, "proj_up")
+    N, R = proj_up.shape
+    out = torch.empty_like(proj_up)
+    if R == 0:
+        return _tag(out, "lora_up")
+    nv.check(nv.lib().svdq_repack_lora_up(proj_up.data_ptr(), out.data_ptr(), N, R, nv.stream_ptr(proj_up.device)))
+    return _tag(out, "lora_up")
+
+
+_REPACKERS = {
+    "qweight": repack_qweight,
+    "wscales": repack_wscales,
+    "vector": repack_vector,
+    "smooth_rcp": repack_smooth,
+    "lora_down": repack_lora_down,
+    "lora_up": repack_lora_up,
+}
+
+# (data_ptr, version, shape, dtype, kind, fp4) -> (weakref to the source, native tensor)
+_cache: dict[tuple, tuple[weakref.ref, torch.Tensor]] = {}
+
+
+def native(t: torch.Tensor | None, kind: str, fp4: bool = False) -> torch.Tensor | None:
+    """Return the native form of ``t``: ``t`` itself when it already is native, else a cached repack
+    of the reference-format tensor (redone when the source is modified or replaced)."""
+    if t is None or is_native(t, kind):
+        return t
+    key = (t.data_ptr(), t._version, tuple(t.shape), t.dtype, kind, fp4)
+    hit = _cache.get(key)
+    if hit is not None and hit[0]() is t:
+        return hit[1]
+    for k in [k for k, (ref, _) in _cache.items() if ref() is None]:
+        del _cache[k]
+    out = _REPACKERS[kind](t, fp4) if kind in ("qweight", "wscales") else _REPACKERS[kind](t)
+    _cache[key] = (weakref.ref(t), out)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# logical views of the kernels' private activation layout (for tests and debugging)
+# ---------------------------------------------------------------------------------------------
+
+
+def act_to_logical(act: torch.Tensor, K: int, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:
+    """Native activation tiles u8 [M_pad, K/2] ([M_pad/32][K/64][32][32 B]) -> one code per element,
+    int8 [M_pad, K] in row/column order.  INT4 signed codes are stored offset-binary (code + 8)."""
+    M_pad = act.shape[0]
+    t = act.reshape(M_pad // 32, K // 64, 32, 32).permute(0, 2, 1, 3).reshape(M_pad, K // 2).to(torch.int16)
+    lo, hi = t & 0xF, (t >> 4) & 0xF
+    codes = torch.stack([lo, hi], dim=-1).reshape(M_pad, K)
+    if not fp4 and not unsigned:
+        codes = codes - 8
+    return codes.to(torch.int8)
+
+
+def logical_to_act(codes: torch.Tensor, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:
+    """Inverse of :func:`act_to_logical` (used by tests to feed hand-made codes to the GEMM)."""
+    M_pad, K = codes.shape
+    c = codes.to(torch.int16)
+    if not fp4 and not unsigned:
+        c = c + 8
+    c = c & 0xF
+    packed = (c[:, 0::2] | (c[:, 1::2] << 4)).to(torch.uint8)
+    return packed.reshape(M_pad // 32, 32, K // 64, 32).permute(0, 2, 1, 3).contiguous().reshape(M_pad, K // 2)

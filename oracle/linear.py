@@ -1,0 +1,130 @@
+"""Logical CPU restatement of the two ops and of the layer built from them.
+
+Test infrastructure only (see ``oracle/__init__.py``).  Everything here works on *logical*
+tensors (no lane permutations, no nibble packing); ``layouts.py`` covers the storage formats.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import quant
+
+
+def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
+    """EpilogueGelu (src/kernels/zgemm/epilogues.cuh:22-44, gemm_utils.cuh:305-312): the tanh form of
+    GELU evaluated in fp32; the library routine is the reference's formula with an exact tanh."""
+    return torch.nn.functional.gelu(x.to(torch.float32), approximate="tanh")
+
+
+def quantize_act_fuse_lora(
+    x: torch.Tensor,
+    proj_down: torch.Tensor,
+    smooth: torch.Tensor | None,
+    fp4: bool = False,
+    pad_size: int = 256,
+):
+    """quantize_w4a4_fuse_lora_kernel (gemm_w4a4.cuh:1097-1184) behind
+    svdq_quantize_w4a4_act_fuse_lora_cuda (nunchaku/ops/quantize.py:11-54).
+
+    x bf16 [M, K]; proj_down bf16 [K, R] (logical); smooth bf16 [K] (logical) or None.
+    Rows M..M_pad are zero-filled by the loader (gemm_base.cuh:591-646) and therefore quantize to
+    code 0 / scale 0 / lora 0.  The low-rank projection uses the raw x (no smoothing):
+    gemm_w4a4.cuh:1159-1171.
+    Returns (codes [M_pad, K], scales [K/G, M_pad], lora_act fp32 [M_pad, R]).
+    """
+    M, K = x.shape
+    M_pad = (M + pad_size - 1) // pad_size * pad_size
+    xp = torch.zeros(M_pad, K, dtype=torch.bfloat16)
+    xp[:M] = x
+    if fp4:
+        codes, scales = quant.quantize_act_nvfp4(xp, smooth)
+    else:
+        codes, scales = quant.quantize_act_int4(xp, smooth, unsigned=False, shift=0.0)
+    lora_act = xp.to(torch.float64) @ proj_down.to(torch.float64)
+    return codes, scales, lora_act.to(torch.float32)
+
+
+def gemm_w4a4(
+    act_deq: torch.Tensor,
+    wgt_deq: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    lora_act_in: torch.Tensor | None = None,
+    lora_up: torch.Tensor | None = None,
+    lora_scales: list[float] | None = None,
+    alpha: float = 1.0,
+    wcscales: torch.Tensor | None = None,
+    gelu: bool = False,
+    silu: bool = False,
+    double: bool = True,
+) -> torch.Tensor:
+    """The GEMM and its epilogue chain on dequantized operands, fp32 (or fp64) accumulated:
+    ``acc = act_deq @ wgt_deq.T`` -> ``* alpha`` (gemm_w4a4.cuh:273-356) -> ``* wcscales + bias``
+    (EpilogueBias, gemm_base.cuh:710-781) -> ``+ bf16(lora_act * scale[r/16]) @ up.T``
+    (EpilogueLoraUp, lora.cuh:110-241) -> GELU / SiLU (epilogues.cuh:22-44, gemm_base.cuh:783-792).
+    Order of the chain: gemm_w4a4_launch_impl.cuh:172-280.  The result is fp32; the caller rounds it
+    to bf16 where the reference stores bf16.
+    """
+    dt = torch.float64 if double else torch.float32
+    acc = act_deq.to(dt) @ wgt_deq.to(dt).t()
+    acc = acc * alpha
+    if wcscales is not None:
+        acc = acc * wcscales.to(dt)[None, :]
+    if bias is not None:
+        acc = acc + bias.to(dt)[None, :]
+    if lora_up is not None:
+        R = lora_up.shape[1]
+        if lora_scales is None:
+            lora_scales = [1.0] * math.ceil(R / 16)
+        sc = torch.tensor([lora_scales[r // 16] if r // 16 < len(lora_scales) else 0.0 for r in range(R)], dtype=torch.float32)
+        a = quant.bf16(lora_act_in.to(torch.float32) * sc[None, :])
+        acc = acc + a.to(dt) @ lora_up.to(dt).t()
+    acc = acc.to(torch.float32)
+    if gelu:
+        acc = gelu_tanh(acc)
+    if silu:
+        acc = acc * torch.sigmoid(acc)
+    return acc
+
+
+class FakeQuantLinear:
+    """Logical-tensor model of SVDQW4A4Linear.forward (nunchaku/models/linear.py:89-132):
+    quantize (+ low-rank down) then GEMM (+ bias, low-rank up).  Also the CPU baseline that the
+    bench times."""
+
+    def __init__(self, wq, ws, smooth, proj_down, proj_up, bias=None, fp4=False, wtscale=1.0, wcscales=None, act_unsigned=False):
+        self.fp4 = fp4
+        self.w_deq = quant.dequant_nvfp4(wq, ws) if fp4 else quant.dequant_int4(wq, ws)
+        self.smooth, self.proj_down, self.proj_up, self.bias = smooth, proj_down, proj_up, bias
+        self.wtscale, self.wcscales, self.act_unsigned = wtscale, wcscales, act_unsigned
+
+    def quantize(self, x):
+        return quantize_act_fuse_lora(x, self.proj_down, self.smooth, fp4=self.fp4)
+
+    def forward_quant(self, codes, scales, lora_act, gelu=False, double=True):
+        a = quant.dequant_nvfp4(codes, scales) if self.fp4 else quant.dequant_int4(codes, scales)
+        return gemm_w4a4(
+            a, self.w_deq, bias=self.bias, lora_act_in=lora_act, lora_up=self.proj_up,
+            alpha=self.wtscale, wcscales=self.wcscales, gelu=gelu, double=double,
+        )
+
+    def forward(self, x, double=True):
+        codes, scales, lora_act = self.quantize(x)
+        return self.forward_quant(codes, scales, lora_act, double=double)[: x.shape[0]]
+
+
+def fused_gelu_mlp(x: torch.Tensor, fc1: FakeQuantLinear, fc2: FakeQuantLinear, double: bool = True):
+    """nunchaku/ops/fused.py:10-47: fc1 GEMM with GELU, then the post-GELU bf16 tile is (a) projected
+    by fc2's down projection and (b) shifted by 0.171875, smoothed and quantized unsigned for fc2
+    (gemm_w4a4_launch_impl.cuh:282-309).  Returns (out fp32 [M, N2], intermediates dict)."""
+    codes, scales, lora_act = fc1.quantize(x)
+    h = quant.bf16(fc1.forward_quant(codes, scales, lora_act, gelu=True, double=double))
+    lora2 = (h.to(torch.float64) @ fc2.proj_down.to(torch.float64)).to(torch.float32)
+    if fc2.fp4:
+        qcodes, qscales = quant.quantize_act_nvfp4(h.to(torch.bfloat16), fc2.smooth)
+    else:
+        qcodes, qscales = quant.quantize_act_int4(h.to(torch.bfloat16), fc2.smooth, unsigned=True, shift=quant.SHIFT_GELU)
+    out = fc2.forward_quant(qcodes, qscales, lora2, double=double)[: x.shape[0]]
+    return out, {"h": h, "qcodes": qcodes, "qscales": qscales, "lora2": lora2}

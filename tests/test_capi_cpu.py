@@ -1,0 +1,134 @@
+"""Host-side checks that need no GPU: the shared library loads, exports every symbol the header
+declares, and rejects bad arguments before launching anything."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from nunchaku_amd import _native as nv
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not nv.LIB_PATH.exists():
+        nv.build()
+    return nv.lib()
+
+
+def test_header_symbols_are_exported(lib):
+    header = (ROOT / "include" / "svdq_amd.h").read_text()
+    declared = set(re.findall(r"^(?:int|const char \*)\s*(svdq_\w+)\(", header, flags=re.M))
+    assert declared == set(nv.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.svdq_abi_version() == nv.SVDQ_ABI_VERSION
+    assert int(re.search(r"#define SVDQ_ABI_VERSION (\d+)", header).group(1)) == nv.SVDQ_ABI_VERSION
+
+
+def test_struct_sizes_match_header_layout():
+    # 6 pointers + 4 int64 + 2 int32 ; 16 pointers + 7 int64 + float + 3 int32
+    assert ctypes.sizeof(nv.QuantizeArgs) == 6 * 8 + 4 * 8 + 2 * 4
+    assert ctypes.sizeof(nv.GemmArgs) == 16 * 8 + 7 * 8 + 4 * 4
+
+
+def test_quantize_rejects_bad_arguments(lib):
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(None, None) == -1
+    a = nv.QuantizeArgs()
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
+    assert b"null" in lib.svdq_last_error()
+    a = nv.QuantizeArgs(input=16, output=16, oscales=16, lora_down=16, lora_act_out=16, M=100, M_pad=200, K=256, R=32)
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
+    assert b"M_pad" in lib.svdq_last_error()
+    a.M_pad = 256
+    a.K = 100
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
+    assert b"K" in lib.svdq_last_error()
+    a.K = 256
+    a.R = 24
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
+    a.R = 32
+    a.input = 8  # misaligned
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
+    assert b"aligned" in lib.svdq_last_error()
+    a.input = 16
+    a.fuse_glu = 1
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -2
+
+
+def test_gemm_rejects_bad_arguments(lib):
+    assert lib.svdq_gemm_w4a4(None, None) == -1
+    a = nv.GemmArgs(act=16, ascales=16, wgt=16, wscales=16, colnorm=16, out=16, M_pad=256, N=128, K=128, M_out=256, N_out=128, alpha=1.0)
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.M_pad = 100
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.N = 100
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.out = None
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.lora_up = 16  # without lora_act_in
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.M_out = 300
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.fuse_silu = 1
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
+
+
+def test_repack_rejects_bad_arguments(lib):
+    assert lib.svdq_repack_qweight(None, None, 128, 128, 0, None) == -1
+    assert lib.svdq_repack_qweight(16, 32, 100, 128, 0, None) == -1
+    assert lib.svdq_repack_qweight(16, 16, 128, 128, 0, None) == -1  # in place
+    assert lib.svdq_repack_wscales(16, 32, 48, 128, 100, None) == -1
+    assert lib.svdq_repack_vector(16, 32, 100, None) == -1
+    assert lib.svdq_repack_smooth(16, 32, 64, None) == -1
+    assert lib.svdq_repack_lora_down(16, 32, 128, 8, None) == -1
+    assert lib.svdq_repack_lora_up(16, 32, 8, 16, None) == -1
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    import torch
+
+    from nunchaku_amd.ops import svdq_gemm_w4a4, svdq_quantize_w4a4_act_fuse_lora
+
+    x = torch.zeros(4, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        svdq_quantize_w4a4_act_fuse_lora(x, lora_down=torch.zeros(128, 16, dtype=torch.bfloat16))
+    with pytest.raises(NotImplementedError):
+        svdq_gemm_w4a4(act=x, wgt=x, rotary_emb=x)
+    with pytest.raises(RuntimeError, match="GPU"):
+        svdq_gemm_w4a4(act=x.view(torch.uint8), wgt=x.view(torch.int8), ascales=x, wscales=x, out=x)
+
+
+def test_module_mirrors_reference_parameters():
+    import torch
+
+    from nunchaku_amd.models.linear import SVDQW4A4Linear
+
+    m = SVDQW4A4Linear(256, 384, rank=32)
+    sd = m.state_dict()
+    # names, shapes and dtypes of nunchaku/models/linear.py:38-72
+    assert {k: (tuple(v.shape), v.dtype) for k, v in sd.items()} == {
+        "qweight": ((384, 128), torch.int8),
+        "bias": ((384,), torch.bfloat16),
+        "wscales": ((4, 384), torch.bfloat16),
+        "smooth_factor": ((256,), torch.bfloat16),
+        "smooth_factor_orig": ((256,), torch.bfloat16),
+        "proj_down": ((256, 32), torch.bfloat16),
+        "proj_up": ((384, 32), torch.bfloat16),
+    }
+    m4 = SVDQW4A4Linear(256, 384, rank=16, precision="nvfp4", bias=False)
+    sd4 = m4.state_dict()
+    assert sd4["wscales"].dtype == torch.float8_e4m3fn and tuple(sd4["wscales"].shape) == (16, 384)
+    assert "wtscale" in sd4 and "wcscales" in sd4 and "bias" not in sd4
+    with pytest.raises(ValueError):
+        SVDQW4A4Linear(256, 384, precision="int8")
+    lin = torch.nn.Linear(256, 384, dtype=torch.bfloat16)
+    assert SVDQW4A4Linear.from_linear(lin, rank=16).rank == 16

@@ -1,0 +1,94 @@
+"""SVDQW4A4Linear end to end on the GPU: reference-format state dict -> load-time repack -> quantize
+-> GEMM, against the oracle, at the CPU-reference configuration and through size-independent
+properties at the FLUX shapes."""
+
+import pytest
+import torch
+
+from conftest import announce
+from gpu_util import check_output, make_module, make_oracle
+from oracle import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config1_full_layer(dev):
+    """M=256, K=N=3072, rank 32, seed 0: the reference's own CPU-runnable case."""
+    from nunchaku_amd import packing
+
+    cfg = synth.CONFIGS["c1"]
+    announce(f"linear config 1 {cfg}")
+    layer = synth.make_layer(cfg["N"], cfg["K"], cfg["R"], seed=cfg["seed"])
+    x = synth.make_activations(cfg["M"], cfg["K"], seed=cfg["seed"])
+    m = make_module(layer, dev)
+    ref = make_oracle(layer)
+    y = m(x.to(dev).view(1, cfg["M"], cfg["K"]))
+    torch.cuda.synchronize()
+    assert y.shape == (1, cfg["M"], cfg["N"]) and y.dtype == torch.bfloat16
+    qx, asc, la = m.quantize(x.to(dev))
+    codes, scales, lora = ref.quantize(x)
+    assert torch.equal(packing.act_to_logical(qx.cpu(), cfg["K"]), codes)
+    assert torch.equal(asc.cpu().view(torch.int16), scales.view(torch.int16))
+    want = ref.forward_quant(codes, scales, lora)[: cfg["M"]]
+    rel = check_output(y[0], want)
+    print(f"config 1 rel-L2 {rel:.2e}")
+
+
+def test_ragged_tokens_3d_input(dev):
+    announce("linear ragged tokens B=2 S=75")
+    layer = synth.make_layer(256, 256, 32, seed=21)
+    x = synth.make_activations(150, 256, seed=21)
+    m = make_module(layer, dev)
+    y = m(x.to(dev).view(2, 75, 256))
+    torch.cuda.synchronize()
+    want = make_oracle(layer).forward(x)
+    check_output(y.reshape(150, 256), want)
+
+
+def test_ops_accept_reference_layout_directly(dev):
+    """nunchaku.ops callers pass checkpoint tensors as they are; they are repacked once and cached."""
+    from nunchaku_amd import packing
+    from nunchaku_amd.ops import svdq_gemm_w4a4, svdq_quantize_w4a4_act_fuse_lora
+
+    announce("ops with reference-layout tensors")
+    layer = synth.make_layer(256, 256, 32, seed=22)
+    sd = {k: v.to(dev) for k, v in synth.to_reference_checkpoint(layer).items()}
+    x = synth.make_activations(256, 256, seed=22)
+    qx, asc, la = svdq_quantize_w4a4_act_fuse_lora(x.to(dev), lora_down=sd["proj_down"], smooth=sd["smooth_factor"])
+    out = torch.empty(256, 256, dtype=torch.bfloat16, device=dev)
+    for _ in range(2):
+        svdq_gemm_w4a4(act=qx, wgt=sd["qweight"], out=out, ascales=asc, wscales=sd["wscales"], lora_act_in=la,
+                       lora_up=sd["proj_up"], bias=sd["bias"])
+    torch.cuda.synchronize()
+    assert len(packing._cache) >= 5
+    check_output(out, make_oracle(layer).forward(x))
+
+
+@pytest.mark.parametrize("name", ["c2_qkv", "c3_fc1"])
+def test_flux_shapes_properties(dev, name):
+    """Full FLUX shapes: bit-exact quantizer against the oracle on a row sample, GEMM checked on a
+    random sample of output rows against the oracle, plus linearity in the bias."""
+    from nunchaku_amd import packing
+
+    cfg = synth.CONFIGS[name]
+    announce(f"linear {name} {cfg}")
+    M, K, N, R = cfg["M"], cfg["K"], cfg["N"], cfg["R"]
+    layer = synth.make_layer(N, K, R, seed=cfg["seed"])
+    x = synth.make_activations(M, K, seed=cfg["seed"])
+    m = make_module(layer, dev)
+    ref = make_oracle(layer)
+    qx, asc, la = m.quantize(x.to(dev))
+    y = m.forward_quant(qx, asc, la)[:M]
+    torch.cuda.synchronize()
+    codes, scales, lora = ref.quantize(x)
+    assert torch.equal(packing.act_to_logical(qx.cpu(), K), codes)
+    assert torch.equal(asc.cpu().view(torch.int16), scales.view(torch.int16))
+    assert (la.cpu() - lora).abs().max().item() <= 2e-5 * lora.abs().max().item()
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(0))[:192]
+    want = ref.forward_quant(codes[rows], scales[:, rows], lora[rows])
+    check_output(y[rows], want)
+    # bias linearity: y(bias) - y(0) == bias up to bf16 rounding of the two outputs
+    m0 = make_module(synth.LogicalLayer(**{**layer.__dict__, "bias": torch.zeros_like(layer.bias)}), dev)
+    y0 = m0.forward_quant(qx, asc, la)[:M]
+    d = (y.float() - y0.float()).cpu() - layer.bias.float()[None, :]
+    assert d.abs().max().item() <= 2 * 2.0**-7 * max(1.0, y.float().abs().max().item())

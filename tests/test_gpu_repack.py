@@ -1,0 +1,80 @@
+"""Load-time repack on the GPU against the oracle's statement of the reference layouts, including
+the golden bytes written by the reference packer."""
+
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+from oracle import layouts as L
+
+pytestmark = pytest.mark.gpu
+GOLD = Path(__file__).parent / "golden" / "packer_vectors.npz"
+
+
+def _bf16(a):
+    return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def test_repack_golden_vectors(dev):
+    from nunchaku_amd import packing
+
+    z = np.load(GOLD)
+    announce("repack golden qweight/wscales/vector/lora N=K=256 R=32")
+    qn = packing.repack_qweight(torch.from_numpy(z["qweight"]).to(dev))
+    N, K = z["codes"].shape
+    # native tiles hold offset-binary codes in row/column order
+    assert torch.equal(packing.act_to_logical(qn.view(torch.uint8).cpu(), K), torch.from_numpy(z["codes"]))
+
+    ws = packing.repack_wscales(_bf16(z["wscales_packed"]).to(dev))
+    logical = _bf16(z["wscales_logical"]).float()
+    back = ws.float().cpu() * ws.colnorm.cpu()[None, :]
+    assert torch.equal(back, logical)  # power-of-two normalisation is exact
+    amax = ws.float().abs().amax(dim=0).cpu()
+    assert ((amax >= 2048) & (amax < 4096)).all()
+
+    v = packing.repack_vector(_bf16(z["vec_packed"].reshape(-1)).to(dev))
+    assert torch.equal(v.cpu().view(torch.int16), _bf16(z["vec_logical"]).view(torch.int16))
+
+    r = packing.repack_smooth(_bf16(z["vec_packed"].reshape(-1)).to(dev))
+    want = (1.0 / _bf16(z["vec_logical"]).float())
+    assert torch.equal(r.cpu(), want)
+
+    up = packing.repack_lora_up(_bf16(z["up_packed"]).to(dev))
+    assert torch.equal(up.cpu().view(torch.int16), _bf16(z["up_logical"]).view(torch.int16))
+
+    dn = packing.repack_lora_down(_bf16(z["down_packed"]).to(dev)).cpu().view(torch.int16)
+    logical = _bf16(z["down_logical"]).view(torch.int16)  # [K, R]
+    R = logical.shape[1]
+    dn = dn.reshape(K // 128, 4, R // 16, 64, 8)
+    c, i, rt, lane, j = np.meshgrid(np.arange(K // 128), np.arange(4), np.arange(R // 16), np.arange(64), np.arange(8), indexing="ij")
+    k = 128 * c + 32 * (lane // 16) + 8 * i + j
+    rk = 16 * rt + lane % 16
+    assert torch.equal(dn, logical[torch.from_numpy(k), torch.from_numpy(rk)])
+
+
+def test_repack_micro_scales(dev):
+    from nunchaku_amd import packing
+
+    z = np.load(GOLD)
+    announce("repack golden nvfp4 micro scales")
+    src = torch.from_numpy(z["mscales_packed"]).view(torch.float8_e4m3fn).to(dev)
+    ws = packing.repack_wscales(src, fp4=True)
+    logical = torch.from_numpy(z["mscales_logical"]).view(torch.float8_e4m3fn).float()
+    assert torch.equal(ws.float().cpu() * ws.colnorm.cpu()[None, :], logical)
+
+
+def test_repack_random_larger(dev):
+    from nunchaku_amd import packing
+
+    rng = np.random.default_rng(5)
+    N, K = 384, 640
+    announce(f"repack random N={N} K={K}")
+    codes = rng.integers(-8, 8, (N, K)).astype(np.int8)
+    qn = packing.repack_qweight(torch.from_numpy(L.pack_qweight(codes)).to(dev))
+    assert torch.equal(packing.act_to_logical(qn.view(torch.uint8).cpu(), K), torch.from_numpy(codes))
+    pat = rng.integers(0, 16, (N, K)).astype(np.int8)
+    qf = packing.repack_qweight(torch.from_numpy(L.pack_qweight(pat)).to(dev), fp4=True)
+    assert torch.equal(packing.act_to_logical(qf.view(torch.uint8).cpu(), K, fp4=True), torch.from_numpy(pat))
