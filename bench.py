@@ -1,0 +1,176 @@
+"""Benchmark of the SVDQuant W4A4 + low-rank linear hot path on one MI355X.
+
+One step = one forward of the layer on inputs already resident in HBM: the quantize + low-rank-down
+kernel followed by the W4A4 GEMM kernel (bias and low-rank up fused).  Workload: FLUX.1-dev MLP fc1,
+M=4608 tokens, K=3072, N=12288, rank 32, INT4 group 64, bf16 in/out, synthetic seeded data.
+
+Prints ONE JSON line:  metric = effective TOPS of the fused layer, (2MNK + 2MR(K+N)) / step time;
+`roofline` describes the GEMM kernel (the dominant one), timed with events on the launch stream;
+`cpu_baseline` is the CPU oracle (PyTorch fake-quant layer) timed on this machine's host cores on a
+bounded row sample of the same layer.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+WORKLOADS = {
+    "flux_mlp_fc1": dict(M=4608, K=3072, N=12288, R=32, seed=2),
+    "flux_qkv": dict(M=4608, K=3072, N=9216, R=32, seed=1),
+    "flux_mlp_fc2": dict(M=4608, K=12288, N=3072, R=32, seed=2),
+    "qwen_batched_r128": dict(M=18432, K=3072, N=12288, R=128, seed=4),
+    "c1_small": dict(M=256, K=3072, N=3072, R=32, seed=0),
+}
+INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, the peak the metric is quoted against
+FP16_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(layer, x, rows: int, iters: int = 3):
+    """The oracle's fake-quant layer on the host cores, on the first `rows` rows of the workload."""
+    import torch
+
+    from oracle import linear as olin
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    ref = olin.FakeQuantLinear(layer.wq, layer.ws, layer.smooth, layer.proj_down, layer.proj_up, layer.bias)
+    xs = x[:rows].contiguous()
+    times = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        y = ref.forward(xs, double=False).to(torch.bfloat16)
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    ops = 2.0 * rows * layer.N * layer.K + 2.0 * rows * layer.R * (layer.K + layer.N)
+    return {
+        "value": ops / t / 1e12, "unit": "TOPS", "cores": cores, "kind": "port",
+        "sample": f"first {rows} of {x.shape[0]} rows of the same layer, fp32 matmul, median of {iters}",
+        "seconds_per_pass": t,
+    }, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="flux_mlp_fc1", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=512)
+    ap.add_argument("--only", choices=["gemm", "quantize"], default=None,
+                    help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from nunchaku_amd.models.linear import SVDQW4A4Linear
+    from oracle import synth
+
+    cfg = WORKLOADS[args.workload]
+    M, K, N, R = cfg["M"], cfg["K"], cfg["N"], cfg["R"]
+    dev = torch.device("cuda:0")
+    layer = synth.make_layer(N, K, R, seed=cfg["seed"])
+    x = synth.make_activations(M, K, seed=cfg["seed"])
+    mod = SVDQW4A4Linear(K, N, rank=R, device=dev)
+    mod.load_state_dict(synth.to_reference_checkpoint(layer))
+    mod.native_tensors()  # load-time repack happens once, outside the timed region
+    xd = x.to(dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    M_pad = (M + 255) // 256 * 256
+    qx = torch.empty(M_pad, K // 2, dtype=torch.uint8, device=dev)
+    asc = torch.empty(K // 64, M_pad, dtype=torch.bfloat16, device=dev)
+    la = torch.empty(M_pad, R, dtype=torch.float32, device=dev)
+    t = mod.native_tensors()
+    from nunchaku_amd.ops import svdq_quantize_w4a4_act_fuse_lora
+
+    def step():
+        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+        mod.forward_quant(qx, asc, la, out)
+
+    if args.only:
+        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            if args.only == "gemm":
+                mod.forward_quant(qx, asc, la, out)
+            else:
+                svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+        torch.cuda.synchronize()
+        print(f"{args.only}: {(time.perf_counter() - t0) * 1e6 / args.steps:.1f} us per launch (host clock, {args.steps} launches)")
+        return
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # whole-step time: exactly `steps` steps between two synchronisations
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-kernel durations with events on the stream the kernels are launched on
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for e in evs:
+        e[0].record()
+        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+        e[1].record()
+        mod.forward_quant(qx, asc, la, out)
+        e[2].record()
+    torch.cuda.synchronize()
+    tq_us = statistics.mean(e[0].elapsed_time(e[1]) for e in evs) * 1e3
+    tg_us = statistics.mean(e[1].elapsed_time(e[2]) for e in evs) * 1e3
+
+    ops_layer = 2.0 * M * N * K + 2.0 * M * R * (K + N)
+    ops_gemm = 2.0 * M * N * K + 2.0 * M * R * N
+    bytes_quant = 2.0 * M * K + M * K / 2 + 2.0 * M * K / 64 + 4.0 * M * R + 2.0 * K * R + 2.0 * K
+    value = ops_layer / (ms_per_step * 1e-3) / 1e12
+    gemm_tops = ops_gemm / (tg_us * 1e-6) / 1e12
+    res = {
+        "metric": "effective TOPS of fused W4A4+LoRA linear at FLUX M=4608; % of MFMA peak",
+        "value": value, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: SVDQW4A4Linear forward M={M} K={K} N={N} rank={R} INT4 g64 bf16 in/out",
+                   "M": M, "K": K, "N": N, "rank": R},
+        "pct_of_int8_mfma_peak": 100.0 * value / INT8_PEAK_TOPS,
+        "us_per_layer": ms_per_step * 1e3,
+        "kernels": {
+            "quantize_fuse_lora_us": tq_us, "gemm_us": tg_us,
+            "quantize_GBps": bytes_quant / (tq_us * 1e-6) / 1e9,
+            "quantize_frac_of_hbm_peak": bytes_quant / (tq_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "gemm_main_term_TOPS": 2.0 * M * N * K / (tg_us * 1e-6) / 1e12,
+        },
+        "roofline": {
+            "kernel": "gemm_w4a4_int4_kernel", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
+            "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": None,
+            "peak_basis": "dense INT8 MFMA (the metric's peak); the kernel issues fp16 MFMA, dense peak 2500",
+            "frac_of_fp16_mfma_peak": gemm_tops / FP16_PEAK_TFLOPS,
+        },
+    }
+    if not args.no_cpu:
+        cb, y_cpu = cpu_baseline(layer, x, min(args.cpu_rows, M))
+        # the same rows from the GPU must agree with the CPU oracle (checker, not the thing measured)
+        got = out[: y_cpu.shape[0]].float().cpu()
+        rel = ((got - y_cpu.float()).norm() / y_cpu.float().norm()).item()
+        cb["gpu_vs_cpu_rel_l2"] = rel
+        res["cpu_baseline"] = cb
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -28,14 +28,16 @@
 // Tiling: workgroup = 4 waves (2 x 2), block tile 256 x 256, wave tile 128 x 128 = 4 x 4 MFMA tiles,
 // 256 fp32 accumulators per lane.  Operand tiles are staged through a 3-deep LDS ring, one k-group
 // per stage; global loads for group g+3 are issued before the math of group g.
-#include "svdq_common.h"
+#include <type_traits>
+
+#include "svdq_quant.h"
 
 using namespace svdq;
 
 namespace {
 
 constexpr int BM = 256, BN = 256;
-constexpr int STAGES = 3;
+constexpr int STAGES = 4;
 constexpr int STAGE_A = 0, STAGE_B = 8192, STAGE_AS = 16384, STAGE_BS = 16384 + 2048;
 constexpr int STAGE_BYTES = 16384 + 4096;  // 8 KB A codes, 8 KB B codes, 2 KB + 2 KB packed scales
 constexpr int OUT_LD = 136;                // bf16 elements per row of the store-staging slab (128 + pad)
@@ -44,7 +46,14 @@ constexpr int ROWMAX_OFF = ROWNORM_OFF + 1024;     // u32 [256] scratch for the 
 constexpr int LDS_BYTES = ROWMAX_OFF + 1024;
 constexpr int NORM_TARGET_EXP = 11;
 
+#ifdef SVDQ_GEMM_TIMING
+#define SVDQ_STAMP(i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 8 + (i)] = __builtin_readcyclecounter()
+#else
+#define SVDQ_STAMP(i)
+#endif
+
 struct GemmParams {
+    long long *stamps;  // debug builds only: per-workgroup phase timestamps
     const uint8_t *act;
     const uint16_t *ascales;
     const uint8_t *wgt;
@@ -55,7 +64,13 @@ struct GemmParams {
     const float *lora_act;
     const uint16_t *lora_up;
     uint16_t *out;
-    int M_pad, N, K, M_out, N_out, R_up;
+    // next-layer fusion
+    uint8_t *qout;               // native activation tiles [M_pad, N/2]
+    void *oscales;               // bf16 [N/64, M_pad] or fp8 [N/16, M_pad]
+    const float *next_smooth_rcp;  // fp32 [N]
+    const bf16x8_t *next_down;   // native proj_down of the next layer ([N, R_down])
+    float *next_lora_out;        // fp32 [M_pad, R_down], zeroed before the launch, accumulated atomically
+    int M_pad, N, K, M_out, N_out, R_up, R_down;
     float alpha;
     float lora_scales[8];
     int gelu;
@@ -64,29 +79,32 @@ struct GemmParams {
 __device__ inline half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 __device__ inline uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
 
-// (a & mask) | magic in one VALU instruction (the compiler otherwise emits an AND and an OR because
-// VOP3 cannot carry 32-bit literals; here the constants live in registers)
-__device__ inline uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) {
-    uint32_t d;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(magic));
-    return d;
-}
+struct DequantConsts {
+    uint32_t magic;   // fp16 pair 1024.0: OR-ing a 4-bit code into its low mantissa bits gives 1024 + u
+    uint32_t mask0, mask4;  // 0x000F000F / 0x00F000F0, kept opaque so that (w & mask) | magic becomes one v_and_or_b32
+    half2_t off1;     // 1024 + 8 (offset-binary signed code in bits 0..3) or 1024 (unsigned)
+    half2_t off16;    // 1024 + 128 (code in bits 4..7) or 1024
+    half2_t woff1, woff16;  // the same for the weight operand (always offset-binary)
+};
 
 // 8 codes of one word -> 8 fp16 values (code - bias) * scale in slot order [0,4,1,5,2,6,3,7]
-template <bool UNSIGNED>
-__device__ inline half8_t dequant_word(uint32_t w, half2_t s, half2_t s16, uint32_t magic) {
-    const half2_t off1 = UNSIGNED ? half2_t{(_Float16)1024.f, (_Float16)1024.f} : half2_t{(_Float16)1032.f, (_Float16)1032.f};
-    const half2_t off16 = UNSIGNED ? half2_t{(_Float16)1024.f, (_Float16)1024.f} : half2_t{(_Float16)1152.f, (_Float16)1152.f};
+__device__ inline half8_t dequant_word(uint32_t w, half2_t s, half2_t s16, const DequantConsts &dc, half2_t off1, half2_t off16) {
     const uint32_t w8 = w >> 8;
-    const half2_t t0 = as_half2(and_or(w, 0x000F000Fu, magic));
-    const half2_t t1 = as_half2(and_or(w, 0x00F000F0u, magic));
-    const half2_t t2 = as_half2(and_or(w8, 0x000F000Fu, magic));
-    const half2_t t3 = as_half2(and_or(w8, 0x00F000F0u, magic));
+    const half2_t t0 = as_half2((w & dc.mask0) | dc.magic);
+    const half2_t t1 = as_half2((w & dc.mask4) | dc.magic);
+    const half2_t t2 = as_half2((w8 & dc.mask0) | dc.magic);
+    const half2_t t3 = as_half2((w8 & dc.mask4) | dc.magic);
     const half2_t a0 = (t0 - off1) * s;
     const half2_t a1 = (t1 - off16) * s16;
     const half2_t a2 = (t2 - off1) * s;
     const half2_t a3 = (t3 - off16) * s16;
     return half8_t{a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
+}
+
+__global__ void zero_f32_kernel(float *p, int64_t n) {
+    const int64_t i = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) * 4;
+    if (i + 3 < n) *(float4_t *)(p + i) = float4_t{0.f, 0.f, 0.f, 0.f};
+    else for (int64_t j = i; j < n; j++) p[j] = 0.f;
 }
 
 __device__ inline float gelu_tanh(float x) {
@@ -100,6 +118,7 @@ __device__ inline float gelu_tanh(float x) {
 
 template <bool ACT_UNSIGNED>
 __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
+    constexpr bool FP4 = false;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -124,6 +143,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
 
     float *rownorm = (float *)(lds + ROWNORM_OFF);
     uint32_t *rowmax = (uint32_t *)(lds + ROWMAX_OFF);
+    SVDQ_STAMP(0);
 
     // ---- prologue: largest activation scale of each of my 256 rows -> power-of-two renormalisation
     rowmax[tid] = 0;
@@ -150,38 +170,53 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
         rownorm[tid] = ldexpf(1.0f, -my_shift);
     }
     const bool col_ok = n0 + tid < p.N;
+    SVDQ_STAMP(1);
 
-    // ---- staging helpers
-    u32x4_t ld_a[2], ld_b[2];
-    uint16_t ld_as;
-    _Float16 ld_bs;
-    const int ca = tid >> 6;
+    // ---- staging -----------------------------------------------------------------------------
+    // Code tiles go global -> LDS with asynchronous 16-byte copies (no registers, no ds_write);
+    // the two scale values per thread travel through registers because they are renormalised on the
+    // way.  All vector-memory traffic of the main loop is issued from volatile asm, in a fixed
+    // order and with a fixed count per iteration, so that one hand-placed s_waitcnt vmcnt(N) per
+    // iteration is exact: group g+4's codes and group g+3's scales are issued at the top of
+    // iteration g; the end of iteration g waits for group g+2 (ten newer operations may stay in
+    // flight), which iteration g+1 reads.  That leaves three iterations for a copy to land.
+    const int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int mt0 = m0 / 32, nt0 = n0 / 32;
-    auto issue_loads = [&](int g) {
+    const uint8_t *a_src[2], *b_src[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int t = ca + 4 * j;
+        const int tb = nt0 + t < ntiles_total ? nt0 + t : ntiles_total - 1;  // clamped: its scales are zero
+        a_src[j] = p.act + (size_t)(mt0 + t) * kgroups * TILE_BYTES + lane * 16;
+        b_src[j] = p.wgt + (size_t)tb * kgroups * TILE_BYTES + lane * 16;
+    }
+    const uint16_t *as_src = p.ascales + m0 + tid;
+    const _Float16 *bs_src = p.wscales + (col_ok ? n0 + tid : p.N - 1);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    auto issue_codes = [&](int g) {  // 4 vector-memory operations
+        const int gc = g < kgroups ? g : kgroups - 1;  // surplus copies at the tail are never consumed
+        const uint32_t dst = lds_base + (g % STAGES) * STAGE_BYTES + ca * TILE_BYTES;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const int t = ca + 4 * j;
-            ld_a[j] = *(const u32x4_t *)(p.act + ((size_t)(mt0 + t) * kgroups + g) * TILE_BYTES + lane * 16);
-            ld_b[j] = (nt0 + t < ntiles_total)
-                          ? *(const u32x4_t *)(p.wgt + ((size_t)(nt0 + t) * kgroups + g) * TILE_BYTES + lane * 16)
-                          : u32x4_t{0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :: "s"(dst + STAGE_A + 4 * j * TILE_BYTES), "v"(a_src[j] + (size_t)gc * TILE_BYTES) : "memory");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(b_src[j] + (size_t)gc * TILE_BYTES) : "memory");
         }
-        ld_as = p.ascales[(size_t)g * p.M_pad + m0 + tid];
-        ld_bs = col_ok ? p.wscales[(size_t)g * p.N + n0 + tid] : (_Float16)0.f;
     };
-    auto store_stage = [&](int st) {
-        uint8_t *base = lds + st * STAGE_BYTES;
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int t = ca + 4 * j;
-            *(u32x4_t *)(base + STAGE_A + t * TILE_BYTES + lane * 16) = ld_a[j];
-            *(u32x4_t *)(base + STAGE_B + t * TILE_BYTES + lane * 16) = ld_b[j];
-        }
-        const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ld_as), my_shift);
+    auto issue_scales = [&](int g, uint32_t &ra, uint32_t &rb) {  // 2 vector-memory operations
+        const int gc = g < kgroups ? g : kgroups - 1;
+        asm volatile("global_load_ushort %0, %1, off" : "=v"(ra) : "v"(as_src + (size_t)gc * p.M_pad) : "memory");
+        asm volatile("global_load_ushort %0, %1, off" : "=v"(rb) : "v"(bs_src + (size_t)gc * p.N) : "memory");
+    };
+    auto store_scales = [&](int g, uint32_t ra, uint32_t rb) {
+        uint8_t *base = lds + (g % STAGES) * STAGE_BYTES;
+        const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), my_shift);
+        const _Float16 sb = col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb) : (_Float16)0.f;
         const _Float16 sa16 = sa * (_Float16)0.0625f;
-        const _Float16 sb16 = ld_bs * (_Float16)0.0625f;
+        const _Float16 sb16 = sb * (_Float16)0.0625f;
         *(u32x2_t *)(base + STAGE_AS + tid * 8) = u32x2_t{as_u32(half2_t{sa, sa}), as_u32(half2_t{sa16, sa16})};
-        *(u32x2_t *)(base + STAGE_BS + tid * 8) = u32x2_t{as_u32(half2_t{ld_bs, ld_bs}), as_u32(half2_t{sb16, sb16})};
+        *(u32x2_t *)(base + STAGE_BS + tid * 8) = u32x2_t{as_u32(half2_t{sb, sb}), as_u32(half2_t{sb16, sb16})};
     };
 
     float16_t acc[4][4];
@@ -192,69 +227,111 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    // prologue: the first STAGES groups; all loads are issued before the first LDS store
+    // prologue: scales of groups 0..2 and codes of groups 0..3
+    uint32_t sa_e, sb_e, sa_o, sb_o;  // scale registers in flight: even / odd groups
     {
-        u32x4_t pa[STAGES][2], pb[STAGES][2];
-        uint16_t pas[STAGES];
-        _Float16 pbs[STAGES];
-#pragma unroll
-        for (int s = 0; s < STAGES; s++) {
-            if (s < kgroups) {
-                issue_loads(s);
-                pa[s][0] = ld_a[0]; pa[s][1] = ld_a[1]; pb[s][0] = ld_b[0]; pb[s][1] = ld_b[1];
-                pas[s] = ld_as; pbs[s] = ld_bs;
-            }
-        }
-#pragma unroll
-        for (int s = 0; s < STAGES; s++) {
-            if (s < kgroups) {
-                ld_a[0] = pa[s][0]; ld_a[1] = pa[s][1]; ld_b[0] = pb[s][0]; ld_b[1] = pb[s][1];
-                ld_as = pas[s]; ld_bs = pbs[s];
-                store_stage(s);
-            }
-        }
+        uint32_t s0a, s0b, s1a, s1b;
+        issue_scales(0, s0a, s0b);
+        issue_scales(1, s1a, s1b);
+        issue_scales(2, sa_e, sb_e);
+        issue_codes(0);
+        issue_codes(1);
+        issue_codes(2);
+        issue_codes(3);
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(s0a), "+v"(s0b), "+v"(s1a), "+v"(s1b), "+v"(sa_e), "+v"(sb_e) :: "memory");
+        store_scales(0, s0a, s0b);
+        store_scales(1, s1a, s1b);
     }
     __syncthreads();
+    SVDQ_STAMP(2);
 
-    uint32_t magic = 0x64006400u;
-    asm volatile("" : "+v"(magic));  // keep the constant in a vector register
-    for (int g = 0; g < kgroups; g++) {
-        const int st = g % STAGES;
-        const bool more = g + STAGES < kgroups;
-        if (more) issue_loads(g + STAGES);
+    // conversion constants, pinned in vector registers (VOP3 cannot take literals, and a scalar
+    // operand on the packed instructions costs a wait state each time)
+    DequantConsts dc;
+    dc.magic = 0x64006400u;
+    dc.off1 = ACT_UNSIGNED ? half2_t{(_Float16)1024.f, (_Float16)1024.f} : half2_t{(_Float16)1032.f, (_Float16)1032.f};
+    dc.off16 = ACT_UNSIGNED ? half2_t{(_Float16)1024.f, (_Float16)1024.f} : half2_t{(_Float16)1152.f, (_Float16)1152.f};
+    dc.woff1 = half2_t{(_Float16)1032.f, (_Float16)1032.f};
+    dc.woff16 = half2_t{(_Float16)1152.f, (_Float16)1152.f};
+    dc.mask0 = 0x000F000Fu;
+    dc.mask4 = 0x00F000F0u;
+    asm volatile("" : "+v"(dc.magic), "+v"(dc.off1), "+v"(dc.off16), "+v"(dc.woff1), "+v"(dc.woff16), "+s"(dc.mask0), "+s"(dc.mask4));
 
+    // Software pipeline over the 16-wide MFMA steps (4 per k-group): while the 16 MFMAs of a step run,
+    // the VALU dequantizes the operands of the next step, so a wave never waits on its own
+    // conversions.  raw_* hold the packed codes and scales of the current k-group, *_n of the next.
+    u32x4_t araw[4], braw[4], araw_n[4], braw_n[4];
+    u32x2_t asc[4], bsc[4], asc_n[4], bsc_n[4];
+    half8_t a0[4], b0[4], a1[4], b1[4];
+    auto read_raw = [&](int st, u32x4_t (&ar)[4], u32x4_t (&br)[4], u32x2_t (&as)[4], u32x2_t (&bs)[4]) {
         const uint8_t *base = lds + st * STAGE_BYTES;
-        u32x4_t araw[4], braw[4];
-        u32x2_t asc[4], bsc[4];
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            araw[t] = *(const u32x4_t *)(base + STAGE_A + (wm * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
-            braw[t] = *(const u32x4_t *)(base + STAGE_B + (wn * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
-            asc[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 8);
-            bsc[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 8);
+            ar[t] = *(const u32x4_t *)(base + STAGE_A + (wm * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
+            br[t] = *(const u32x4_t *)(base + STAGE_B + (wn * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
+            as[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 8);
+            bs[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 8);
         }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            half8_t a[4], b[4];
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                a[t] = dequant_word<ACT_UNSIGNED>(araw[t][i], as_half2(asc[t][0]), as_half2(asc[t][1]), magic);
-                b[t] = dequant_word<false>(braw[t][i], as_half2(bsc[t][0]), as_half2(bsc[t][1]), magic);
-            }
-#pragma unroll
-            for (int mt = 0; mt < 4; mt++)
-#pragma unroll
-                for (int nt = 0; nt < 4; nt++)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], acc[mt][nt], 0, 0, 0);
-        }
-        __syncthreads();
-        if (more) store_stage(st);
+    };
+#define SVDQ_CONVERT(AR, BR, AS, BS, I, A, B)                                                             \
+    _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                       \
+        A[t] = dequant_word(AR[t][I], as_half2(AS[t][0]), as_half2(AS[t][1]), dc, dc.off1, dc.off16);       \
+        B[t] = dequant_word(BR[t][I], as_half2(BS[t][0]), as_half2(BS[t][1]), dc, dc.woff1, dc.woff16);              \
     }
-    __syncthreads();
+#define SVDQ_MFMA(A, B)                                                                                   \
+    _Pragma("unroll") for (int mt = 0; mt < 4; mt++) _Pragma("unroll") for (int nt = 0; nt < 4; nt++)     \
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[mt], B[nt], acc[mt][nt], 0, 0, 0);
+    // one k-group; S_USE holds the scales of group G+2 (issued one iteration ago), S_LOAD receives G+3's
+#define SVDQ_GROUP(G, SA_USE, SB_USE, SA_LOAD, SB_LOAD)                                                   \
+    {                                                                                                     \
+        issue_scales((G) + 3, SA_LOAD, SB_LOAD);                                                          \
+        issue_codes((G) + 4);                                                                             \
+        SVDQ_CONVERT(araw, braw, asc, bsc, 1, a1, b1)                                                     \
+        SVDQ_MFMA(a0, b0)                                                                                 \
+        SVDQ_CONVERT(araw, braw, asc, bsc, 2, a0, b0)                                                     \
+        SVDQ_MFMA(a1, b1)                                                                                 \
+        read_raw(((G) + 1) % STAGES, araw_n, braw_n, asc_n, bsc_n);                                       \
+        SVDQ_CONVERT(araw, braw, asc, bsc, 3, a1, b1)                                                     \
+        SVDQ_MFMA(a0, b0)                                                                                 \
+        SVDQ_CONVERT(araw_n, braw_n, asc_n, bsc_n, 0, a0, b0)                                             \
+        SVDQ_MFMA(a1, b1)                                                                                 \
+        _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                   \
+            araw[t] = araw_n[t]; braw[t] = braw_n[t]; asc[t] = asc_n[t]; bsc[t] = bsc_n[t];               \
+        }                                                                                                 \
+        /* an MFMA takes two issue slots, every other instruction one; 8 passes cover six of them */      \
+        _Pragma("unroll") for (int k = 0; k < 32; k++) {                                                  \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
+            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);                                            \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
+        }                                                                                                 \
+        asm volatile("s_waitcnt vmcnt(10)" : "+v"(SA_USE), "+v"(SB_USE) :: "memory");                     \
+        store_scales((G) + 2, SA_USE, SB_USE);                                                            \
+        __syncthreads();                                                                                  \
+    }
 
-    // ---- epilogue, one 32-row slab (mt) of the wave tile at a time ------------------------------
+    read_raw(0, araw, braw, asc, bsc);
+    SVDQ_CONVERT(araw, braw, asc, bsc, 0, a0, b0)
+    for (int g = 0; g < kgroups; g += 2) {  // K is a multiple of 128: an even number of groups
+        SVDQ_GROUP(g, sa_e, sb_e, sa_o, sb_o)
+        SVDQ_GROUP(g + 1, sa_o, sb_o, sa_e, sb_e)
+    }
+#undef SVDQ_GROUP
+#undef SVDQ_CONVERT
+#undef SVDQ_MFMA
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // pin the accumulators in the accumulation registers across the loop exit: without this the
+    // register allocator may place the 256 copies into ordinary registers inside the loop body
+    asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]),
+                      "+a"(acc[1][2]), "+a"(acc[1][3]), "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]),
+                      "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
+    __syncthreads();
+    SVDQ_STAMP(3);
+
+    // ---- epilogue -----------------------------------------------------------------------------
     // accumulator element e of tile (mt, nt): row 8*(e/4) + 4*h + e%4, column r32 of the tile
     const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
+    // per-column factor (undoes the column normalisation, applies alpha and wcscales) and bias
     float colf[4], biasf[4];
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
@@ -265,10 +342,55 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
         colf[nt] = cf;
         biasf[nt] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
     }
-    uint16_t *slab = (uint16_t *)(lds + wave * (32 * OUT_LD * 2));
+    // operands of the low-rank up projection for the first 32 ranks, requested in one batch so that
+    // their latency is paid once (further ranks are fetched inside the slab loop)
     const int nsteps = p.R_up / 16;
+    bf16x8_t la_pre[4][2], lb_pre[4][2];
+    auto load_la = [&](int mt, int s) {
+        const float ls = p.lora_scales[s < 8 ? s : 7];
+        const float4_t *ap = (const float4_t *)(p.lora_act + (size_t)(wrow0 + mt * 32 + r32) * p.R_up + 16 * s + 8 * h);
+        const float4_t v0 = ap[0], v1 = ap[1];
+        u32x4_t w;
+        w[0] = f32_to_bf16_bits(v0[0] * ls) | (f32_to_bf16_bits(v0[1] * ls) << 16);
+        w[1] = f32_to_bf16_bits(v0[2] * ls) | (f32_to_bf16_bits(v0[3] * ls) << 16);
+        w[2] = f32_to_bf16_bits(v1[0] * ls) | (f32_to_bf16_bits(v1[1] * ls) << 16);
+        w[3] = f32_to_bf16_bits(v1[2] * ls) | (f32_to_bf16_bits(v1[3] * ls) << 16);
+        return __builtin_bit_cast(bf16x8_t, w);
+    };
+    auto load_lb = [&](int nt, int s) {
+        const int n = wcol0 + nt * 32 + r32;
+        const u32x4_t bw = n < p.N ? *(const u32x4_t *)(p.lora_up + (size_t)n * p.R_up + 16 * s + 8 * h) : u32x4_t{0, 0, 0, 0};
+        return __builtin_bit_cast(bf16x8_t, bw);
+    };
+    if (nsteps > 0) {
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++) {
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int s = k < nsteps ? k : 0;
+                la_pre[t][k] = load_la(t, s);
+                lb_pre[t][k] = load_lb(t, s);
+            }
+    }
+
+    // reciprocal smoothing factors of the next layer for the 32 columns this lane quantizes
+    // (work item of the quantizing pass: row = item / 4, 32-column quarter = item % 4 = lane % 4)
+    float nrs[32];
+    if (p.qout) {
+        const float4_t *sp = (const float4_t *)(p.next_smooth_rcp + (wcol0 < p.N ? wcol0 : 0) + (lane & 3) * 32);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float4_t v = sp[i];
+            nrs[4 * i] = v[0]; nrs[4 * i + 1] = v[1]; nrs[4 * i + 2] = v[2]; nrs[4 * i + 3] = v[3];
+        }
+    }
+    uint16_t *slab = (uint16_t *)(lds + wave * (32 * OUT_LD * 2));
+    const int ngroups_out = p.N / 64;
+    // one 32-row slab of the wave tile; instantiated four times with a compile-time slab index (a
+    // pragma-unrolled loop of this size is refused by the unroller, which would push the
+    // accumulators into scratch memory)
+    auto slab_epilogue = [&](auto MT) {
+        constexpr int mt = decltype(MT)::value;
         // undo the power-of-two normalisation; per-channel scale and bias (EpilogueBias, gemm_base.cuh:710-781)
 #pragma unroll
         for (int e = 0; e < 16; e++) {
@@ -277,21 +399,19 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
             for (int nt = 0; nt < 4; nt++) acc[mt][nt][e] = acc[mt][nt][e] * rn * colf[nt] + biasf[nt];
         }
         // low-rank up projection: acc += bf16(lora_act * scale) @ up^T   (lora.cuh:110-241)
-        for (int s = 0; s < nsteps; s++) {
-            const float ls = p.lora_scales[s < 8 ? s : 7];
-            const float4_t *ap = (const float4_t *)(p.lora_act + (size_t)(wrow0 + mt * 32 + r32) * p.R_up + 16 * s + 8 * h);
-            const float4_t v0 = ap[0], v1 = ap[1];
-            u32x4_t w;
-            w[0] = f32_to_bf16_bits(v0[0] * ls) | (f32_to_bf16_bits(v0[1] * ls) << 16);
-            w[1] = f32_to_bf16_bits(v0[2] * ls) | (f32_to_bf16_bits(v0[3] * ls) << 16);
-            w[2] = f32_to_bf16_bits(v1[0] * ls) | (f32_to_bf16_bits(v1[1] * ls) << 16);
-            w[3] = f32_to_bf16_bits(v1[2] * ls) | (f32_to_bf16_bits(v1[3] * ls) << 16);
-            const bf16x8_t la = __builtin_bit_cast(bf16x8_t, w);
+        if (nsteps > 0) {
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) {
-                const int n = wcol0 + nt * 32 + r32;
-                const u32x4_t bw = n < p.N ? *(const u32x4_t *)(p.lora_up + (size_t)n * p.R_up + 16 * s + 8 * h) : u32x4_t{0, 0, 0, 0};
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(la, __builtin_bit_cast(bf16x8_t, bw), acc[mt][nt], 0, 0, 0);
+            for (int k = 0; k < 2; k++)
+                if (k < nsteps) {
+#pragma unroll
+                    for (int nt = 0; nt < 4; nt++)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(la_pre[mt][k], lb_pre[nt][k], acc[mt][nt], 0, 0, 0);
+                }
+            for (int s2 = 2; s2 < nsteps; s2++) {
+                const bf16x8_t la = load_la(mt, s2);
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(la, load_lb(nt, s2), acc[mt][nt], 0, 0, 0);
             }
         }
         if (p.gelu) {
@@ -300,7 +420,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[mt][nt][e] = gelu_tanh(acc[mt][nt][e]);
         }
-        // bf16 tile -> per-wave LDS slab (32 rows x 128 columns) -> 16-byte row-contiguous global stores
+        // bf16 tile -> per-wave LDS slab (32 rows x 128 columns): every later consumer reads whole rows
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
 #pragma unroll
@@ -308,7 +428,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
                 slab[(8 * (e / 4) + 4 * h + (e % 4)) * OUT_LD + nt * 32 + r32] = (uint16_t)f32_to_bf16_bits(acc[mt][nt][e]);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (p.out) {
+        if (p.out) {  // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores
 #pragma unroll
             for (int pass = 0; pass < 8; pass++) {
                 const int rr = pass * 4 + (lane >> 4), cc = (lane & 15) * 8;
@@ -316,9 +436,77 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
                 if (m < p.M_out && n < p.N_out) *(u32x4_t *)(p.out + (size_t)m * p.N_out + n) = *(const u32x4_t *)(slab + rr * OUT_LD + cc);
             }
         }
+        if (p.next_down && wcol0 < p.N) {
+            // low-rank down projection of the next layer on the bf16 tile (EpilogueLoraDown,
+            // lora.cuh:243-353): this wave's 128 columns are one 128-chunk of the next layer's K
+            const int RT = p.R_down / 16;
+            const int r16 = lane & 15, q = lane >> 4;
+            for (int rt = 0; rt < RT; rt++) {
+                float4_t d[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const bf16x8_t b = p.next_down[((size_t)((wcol0 / 128) * 4 + i) * RT + rt) * 64 + lane];
+#pragma unroll
+                    for (int m2 = 0; m2 < 2; m2++) {
+                        const bf16x8_t a = *(const bf16x8_t *)(slab + (16 * m2 + r16) * OUT_LD + 32 * q + 8 * i);
+                        d[m2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, d[m2], 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int m2 = 0; m2 < 2; m2++)
+#pragma unroll
+                    for (int i2 = 0; i2 < 4; i2++)
+                        atomicAdd(p.next_lora_out + (size_t)(wrow0 + mt * 32 + 16 * m2 + 4 * q + i2) * p.R_down + 16 * rt + r16, d[m2][i2]);
+            }
+        }
+        if (p.qout && wcol0 < p.N) {
+            // EpilogueQuantize (gemm_w4a4.cuh:930-1043): shift, smooth, quantize for the next layer
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++) {
+                const int item = pass * 64 + lane;
+                const int rr = item >> 2, qc = item & 3;
+                const u32x4_t *sp = (const u32x4_t *)(slab + rr * OUT_LD + qc * 32);
+                float y[32];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const u32x4_t v = sp[i];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float lo = bits_f32(v[j] << 16), hi = bits_f32(v[j] & 0xFFFF0000u);
+                        if (!FP4) {  // INT4 next layer: unsigned codes after a +0.171875 shift (launch_impl.cuh:286-294)
+                            lo = bf16_bits_to_f32(f32_to_bf16_bits(__fadd_rn(lo, 0.171875f)));
+                            hi = bf16_bits_to_f32(f32_to_bf16_bits(__fadd_rn(hi, 0.171875f)));
+                        }
+                        y[8 * i + 2 * j] = smooth_quotient(lo, nrs[8 * i + 2 * j]);
+                        y[8 * i + 2 * j + 1] = smooth_quotient(hi, nrs[8 * i + 2 * j + 1]);
+                    }
+                }
+                const int m = wrow0 + mt * 32 + rr;
+                const int gidx = (wcol0 + qc * 32) / 64;
+                u32x4_t words;
+                if (!FP4) {
+                    float sc;
+                    quantize_int4_half_group<true>(y, 1, words, sc);
+                    if ((qc & 1) == 0) ((uint16_t *)p.oscales)[(size_t)gidx * p.M_pad + m] = (uint16_t)f32_to_bf16_bits(sc);
+                } else {
+                    uint32_t sc[2];
+                    quantize_nvfp4_two_groups(y, words, sc);
+                    uint8_t *os = (uint8_t *)p.oscales;
+                    const int g16 = (wcol0 + qc * 32) / 16;
+                    os[(size_t)g16 * p.M_pad + m] = (uint8_t)sc[0];
+                    os[(size_t)(g16 + 1) * p.M_pad + m] = (uint8_t)sc[1];
+                }
+                *(u32x4_t *)(p.qout + ((size_t)(m / 32) * ngroups_out + gidx) * TILE_BYTES + (m % 32) * 32 + 16 * (qc & 1)) = words;
+            }
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-    }
+    };
+    slab_epilogue(std::integral_constant<int, 0>{});
+    slab_epilogue(std::integral_constant<int, 1>{});
+    slab_epilogue(std::integral_constant<int, 2>{});
+    slab_epilogue(std::integral_constant<int, 3>{});
+    SVDQ_STAMP(4);
 }
 
 }  // namespace
@@ -344,9 +532,20 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     SVDQ_REQUIRE(a->M_pad * a->N < (1ll << 40) && a->K < (1 << 24), "gemm: shape too large");
     if (a->fuse_silu) return fail(SVDQ_EUNSUPPORTED, "gemm: fuse_silu is not implemented");
     if (a->fp4) return fail(SVDQ_EUNSUPPORTED, "gemm: NVFP4 operands are not implemented yet");
-    if (a->qout) return fail(SVDQ_EUNSUPPORTED, "gemm: next-layer quantization epilogue is not implemented yet");
+    if (a->qout) {
+        SVDQ_REQUIRE(a->oscales && a->next_smooth_rcp, "gemm: qout needs oscales and next_smooth_rcp");
+        SVDQ_REQUIRE(((uintptr_t)a->qout | (uintptr_t)a->next_smooth_rcp) % 16 == 0, "gemm: qout pointers must be 16-byte aligned");
+    }
+    SVDQ_REQUIRE((a->next_lora_down != nullptr) == (a->next_lora_act_out != nullptr) && (a->next_lora_down != nullptr) == (a->R_down > 0),
+                 "gemm: next_lora_down, next_lora_act_out and R_down go together");
+    SVDQ_REQUIRE(a->R_down >= 0 && a->R_down % 16 == 0 && a->R_down <= 128, "gemm: R_down (%lld) must be a multiple of 16, at most 128", (long long)a->R_down);
 
     GemmParams p;
+#ifdef SVDQ_GEMM_TIMING
+    p.stamps = (long long *)a->next_lora_act_out;  // debug builds borrow this slot for the stamp buffer
+#else
+    p.stamps = nullptr;
+#endif
     p.act = (const uint8_t *)a->act;
     p.ascales = (const uint16_t *)a->ascales;
     p.wgt = (const uint8_t *)a->wgt;
@@ -357,16 +556,29 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     p.lora_act = a->lora_act_in;
     p.lora_up = (const uint16_t *)a->lora_up;
     p.out = (uint16_t *)a->out;
+    p.qout = (uint8_t *)a->qout;
+    p.oscales = a->oscales;
+    p.next_smooth_rcp = a->next_smooth_rcp;
+    p.next_down = (const bf16x8_t *)a->next_lora_down;
+    p.next_lora_out = a->next_lora_act_out;
+    p.R_down = (int)a->R_down;
     p.M_pad = (int)a->M_pad; p.N = (int)a->N; p.K = (int)a->K;
     p.M_out = (int)a->M_out; p.N_out = (int)a->N_out; p.R_up = (int)a->R_up;
     p.alpha = a->alpha;
     for (int i = 0; i < 8; i++) p.lora_scales[i] = (a->lora_scales && i < (a->R_up + 15) / 16) ? a->lora_scales[i] : 1.0f;
-    p.gelu = 0;
+    p.gelu = a->qout != nullptr;  // the GELU is composed exactly when the next layer's input is produced (launch_impl.cuh:282-309)
+#ifdef SVDQ_GEMM_TIMING
+    p.next_down = nullptr; p.next_lora_out = nullptr; p.R_down = 0;
+#endif
 
     const int nwg = (int)(a->M_pad / BM) * (int)((a->N + BN - 1) / BN);
     auto kern = a->act_unsigned ? gemm_w4a4_int4_kernel<true> : gemm_w4a4_int4_kernel<false>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+    if (p.next_lora_out) {  // the low-rank projection for the next layer is accumulated across column blocks
+        const int64_t n = a->M_pad * a->R_down;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, p.next_lora_out, n);
+    }
     hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), LDS_BYTES, (hipStream_t)stream, p);
     return check_launch("gemm_w4a4");
 }

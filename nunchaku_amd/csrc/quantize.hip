@@ -18,58 +18,11 @@
 //   code = clamp(rne(y * r), -8, 7)               (gemm_w4a4.cuh:429-523)
 //   NVFP4: s = min(f32(amax) * fl32(1/6), 448), stored e4m3(s), code = e2m1(y * fl32(1/s))
 //                                                  (gemm_w4a4.cuh:85-187)
-#include "svdq_common.h"
+#include "svdq_quant.h"
 
 using namespace svdq;
 
 namespace {
-
-constexpr float RECIP_7 = 1.0f / 7.0f;
-constexpr float RECIP_15 = 1.0f / 15.0f;
-constexpr float RECIP_6 = 1.0f / 6.0f;
-constexpr float RNE_MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds to an integer (RNE)
-
-__device__ inline float smooth_quotient(float x, float rcp) {
-    // bf16(x / smooth) as fp32, see the header comment
-    return bf16_bits_to_f32(f32_to_bf16_bits(__fmul_rn(x, rcp)));
-}
-
-// 8 clamped-and-rounded codes (already offset so that they are in [0, 15]) -> one word
-__device__ inline uint32_t pack8(const float (&v)[8]) {
-    uint32_t w = 0;
-#pragma unroll
-    for (int j = 0; j < 8; j++) w |= (f32_bits(v[j]) & 15u) << (4 * j);
-    return w;
-}
-
-// fp32 (finite, >= 0, <= 448) -> e4m3 bit pattern, round to nearest even
-__device__ inline uint32_t f32_to_e4m3(float s) {
-    if (s < 0.0009765625f) return 0;  // below half of the smallest subnormal (2^-10) rounds to 0
-    if (s < 0.015625f) {              // subnormal range: multiples of 2^-9
-        float t = __fadd_rn(__fmul_rn(s, 512.0f), RNE_MAGIC);
-        return f32_bits(t) & 0xFF;    // 0..8 (8 == smallest normal, pattern 0x08)
-    }
-    uint32_t b = f32_bits(s);
-    b += 0x7FFFFu + ((b >> 20) & 1u);  // round mantissa to 3 bits, ties to even
-    const int ex = (int)(b >> 23) - 127 + 7;
-    return (uint32_t)(ex << 3) | ((b >> 20) & 7u);
-}
-
-// fp32 -> 4-bit e2m1 pattern, round to nearest even, saturating at 6
-__device__ inline uint32_t f32_to_e2m1(float v) {
-    const float a = fabsf(v);
-    uint32_t c;
-    // grid 0 .5 1 1.5 2 3 4 6 ; ties go to the pattern with an even low bit
-    if (a <= 0.25f) c = 0;
-    else if (a < 0.75f) c = 1;
-    else if (a <= 1.25f) c = 2;
-    else if (a < 1.75f) c = 3;
-    else if (a <= 2.5f) c = 4;
-    else if (a < 3.5f) c = 5;
-    else if (a <= 5.0f) c = 6;
-    else c = 7;
-    return c | ((f32_bits(v) >> 28) & 8u);
-}
 
 struct QuantParams {
     const uint16_t *x;       // bf16 [M, K]
@@ -155,43 +108,13 @@ __global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) 
             uint8_t *dst = p.act + tile * TILE_BYTES + (row % 32) * 32 + 16 * (q & 1);
             u32x4_t words;
             if (!FP4) {
-                float amax = 0.f;
-#pragma unroll
-                for (int e = 0; e < 32; e++) amax = fmaxf(amax, fabsf(y[e]));
-                amax = fmaxf(amax, __shfl_xor(amax, 16));
-                const float s = __fmul_rn(amax, RECIP_7);
-                const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
-#pragma unroll
-                for (int wi = 0; wi < 4; wi++) {
-                    float v[8];
-#pragma unroll
-                    for (int j = 0; j < 8; j++) {
-                        float t = __fmul_rn(y[8 * wi + j], rcp);
-                        t = fminf(fmaxf(t, -8.0f), 7.0f);
-                        v[j] = __fadd_rn(t, RNE_MAGIC + 8.0f);  // offset-binary code in the low nibble
-                    }
-                    words[wi] = pack8(v);
-                }
+                float s;
+                quantize_int4_half_group<false>(y, 16, words, s);
                 if ((q & 1) == 0)
                     ((uint16_t *)p.oscales)[(size_t)(2 * c + (q >> 1)) * p.M_pad + row] = (uint16_t)f32_to_bf16_bits(s);
             } else {
                 uint32_t sc[2];
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    float amax = 0.f;
-#pragma unroll
-                    for (int e = 0; e < 16; e++) amax = fmaxf(amax, fabsf(y[16 * h + e]));
-                    const float s = fminf(__fmul_rn(amax, RECIP_6), 448.0f);
-                    const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
-                    sc[h] = f32_to_e4m3(s);
-#pragma unroll
-                    for (int wi = 0; wi < 2; wi++) {
-                        uint32_t w = 0;
-#pragma unroll
-                        for (int j = 0; j < 8; j++) w |= f32_to_e2m1(s > 0.f ? __fmul_rn(y[16 * h + 8 * wi + j], rcp) : 0.f) << (4 * j);
-                        words[2 * h + wi] = w;
-                    }
-                }
+                quantize_nvfp4_two_groups(y, words, sc);
                 uint8_t *os = (uint8_t *)p.oscales;
                 os[(size_t)(8 * c + 2 * q) * p.M_pad + row] = (uint8_t)sc[0];
                 os[(size_t)(8 * c + 2 * q + 1) * p.M_pad + row] = (uint8_t)sc[1];

@@ -1,0 +1,110 @@
+// Device-side core of the 4-bit activation quantizers, shared by the stand-alone quantize kernel and
+// by the GEMM epilogue that quantizes for the next layer.  Arithmetic contract (IEEE fp32,
+// round-to-nearest-even, no contraction), following src/kernels/zgemm/gemm_w4a4.cuh:429-523 (INT4) and
+// :85-187 (NVFP4):
+//   amax = max |y| over the group (y are bf16 values held as fp32)
+//   INT4 : s = amax * fl32(1/7) (signed) or fl32(1/15) (unsigned); stored scale bf16(s);
+//          code = clamp(rne(y * fl32(1/s)), lo, hi); a zero group gives codes 0 and scale 0
+//   NVFP4: s = min(amax * fl32(1/6), 448); stored scale e4m3(s); code = e2m1(y * fl32(1/s))
+#pragma once
+
+#include "svdq_common.h"
+
+namespace svdq {
+
+constexpr float RECIP_7 = 1.0f / 7.0f;
+constexpr float RECIP_15 = 1.0f / 15.0f;
+constexpr float RECIP_6 = 1.0f / 6.0f;
+constexpr float RNE_MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds to an integer (RNE)
+
+__device__ inline float smooth_quotient(float x, float rcp) {
+    // bf16(x / smooth) as fp32, see the header comment
+    return bf16_bits_to_f32(f32_to_bf16_bits(__fmul_rn(x, rcp)));
+}
+
+// 8 clamped-and-rounded codes (already offset so that they are in [0, 15]) -> one word
+__device__ inline uint32_t pack8(const float (&v)[8]) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) w |= (f32_bits(v[j]) & 15u) << (4 * j);
+    return w;
+}
+
+// fp32 (finite, >= 0, <= 448) -> e4m3 bit pattern, round to nearest even
+__device__ inline uint32_t f32_to_e4m3(float s) {
+    if (s < 0.0009765625f) return 0;  // below half of the smallest subnormal (2^-10) rounds to 0
+    if (s < 0.015625f) {              // subnormal range: multiples of 2^-9
+        float t = __fadd_rn(__fmul_rn(s, 512.0f), RNE_MAGIC);
+        return f32_bits(t) & 0xFF;    // 0..8 (8 == smallest normal, pattern 0x08)
+    }
+    uint32_t b = f32_bits(s);
+    b += 0x7FFFFu + ((b >> 20) & 1u);  // round mantissa to 3 bits, ties to even
+    const int ex = (int)(b >> 23) - 127 + 7;
+    return (uint32_t)(ex << 3) | ((b >> 20) & 7u);
+}
+
+// fp32 -> 4-bit e2m1 pattern, round to nearest even, saturating at 6
+__device__ inline uint32_t f32_to_e2m1(float v) {
+    const float a = fabsf(v);
+    uint32_t c;
+    // grid 0 .5 1 1.5 2 3 4 6 ; ties go to the pattern with an even low bit
+    if (a <= 0.25f) c = 0;
+    else if (a < 0.75f) c = 1;
+    else if (a <= 1.25f) c = 2;
+    else if (a < 1.75f) c = 3;
+    else if (a <= 2.5f) c = 4;
+    else if (a < 3.5f) c = 5;
+    else if (a <= 5.0f) c = 6;
+    else c = 7;
+    return c | ((f32_bits(v) >> 28) & 8u);
+}
+
+
+// One lane holds 32 consecutive elements of a row = half of a 64-group; the other half lives in the
+// lane `partner_xor` away.  Produces the 16 bytes of codes of this half and the group scale.
+// Signed codes are emitted offset-binary (code + 8), unsigned ones as they are.
+template <bool UNSIGNED>
+__device__ inline void quantize_int4_half_group(const float (&y)[32], int partner_xor, u32x4_t &words, float &scale) {
+    float amax = 0.f;
+#pragma unroll
+    for (int e = 0; e < 32; e++) amax = fmaxf(amax, fabsf(y[e]));
+    amax = fmaxf(amax, __shfl_xor(amax, partner_xor));
+    const float s = __fmul_rn(amax, UNSIGNED ? RECIP_15 : RECIP_7);
+    const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
+    const float lo = UNSIGNED ? 0.0f : -8.0f, hi = UNSIGNED ? 15.0f : 7.0f;
+    const float magic = UNSIGNED ? RNE_MAGIC : RNE_MAGIC + 8.0f;
+#pragma unroll
+    for (int wi = 0; wi < 4; wi++) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            float t = __fmul_rn(y[8 * wi + j], rcp);
+            t = fminf(fmaxf(t, lo), hi);
+            v[j] = __fadd_rn(t, magic);  // the rounded code sits in the low nibble of the bit pattern
+        }
+        words[wi] = pack8(v);
+    }
+    scale = s;
+}
+
+// One lane holds two whole 16-groups.  Produces 16 bytes of E2M1 patterns and the two E4M3 scales.
+__device__ inline void quantize_nvfp4_two_groups(const float (&y)[32], u32x4_t &words, uint32_t (&sc)[2]) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        float amax = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; e++) amax = fmaxf(amax, fabsf(y[16 * h + e]));
+        const float s = fminf(__fmul_rn(amax, RECIP_6), 448.0f);
+        const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
+        sc[h] = f32_to_e4m3(s);
+#pragma unroll
+        for (int wi = 0; wi < 2; wi++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int j = 0; j < 8; j++) w |= f32_to_e2m1(s > 0.f ? __fmul_rn(y[16 * h + 8 * wi + j], rcp) : 0.f) << (4 * j);
+            words[2 * h + wi] = w;
+        }
+    }
+}
+
+}  // namespace svdq
