@@ -57,8 +57,9 @@ int svdq_repack_qweight(const void *src, void *dst, int64_t N, int64_t K, int fp
  * Replaces packed_wscale_t loads, gemm_base.cuh:474-489. */
 int svdq_repack_wscales(const void *src, void *dst_scales, void *dst_colnorm, int64_t N, int64_t K, void *stream);
 
-/* NVFP4 micro scales fp8-e4m3 [K/16, N] (reference lane order) -> native fp16 [K/16, N] and fp32
- * colnorm [N], normalised as above.  Replaces packed_wmscale_t loads, gemm_w4a4.cuh:75-83. */
+/* NVFP4 micro scales fp8-e4m3 [K/16, N] (reference lane order) -> native fp16 [K/64][N][4] (the four
+ * 16-groups of a 64-wide k tile side by side) and fp32 colnorm [N], normalised as above.
+ * Replaces packed_wmscale_t loads, gemm_w4a4.cuh:75-83. */
 int svdq_repack_wmscales(const void *src, void *dst_scales, void *dst_colnorm, int64_t N, int64_t K, void *stream);
 
 /* bias / smooth_factor / wcscales bf16 [N] (reference lane order) -> bf16 [N] in channel order.
@@ -85,7 +86,8 @@ typedef struct svdq_quantize_args {
     const void *input;      /* bf16 [M, K] row-major */
     void *output;           /* u8 [M_pad, K/2] native activation tiles [M_pad/32][K/G64][32][32 B];
                                INT4 codes offset-binary (code + 8), NVFP4 patterns unchanged      */
-    void *oscales;          /* INT4: bf16 [K/64, M_pad]; NVFP4: fp8-e4m3 [K/16, M_pad]; group-major */
+    void *oscales;          /* INT4: bf16 [K/64][M_pad]; NVFP4: fp8-e4m3, K/16 * M_pad values stored as
+                               [K/64][M_pad][4] (four 16-groups of a 64-group side by side)      */
     const void *lora_down;  /* native proj_down (svdq_repack_lora_down) or NULL when R == 0       */
     float *lora_act_out;    /* fp32 [M_pad, R] row-major; fully written (no pre-zero needed)       */
     const float *smooth_rcp;/* fp32 [K] from svdq_repack_smooth, or NULL for no smoothing          */
@@ -106,7 +108,7 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * ------------------------------------------------------------------------------------------ */
 typedef struct svdq_gemm_args {
     const void *act;        /* u8 native activation tiles [M_pad, K/2]                              */
-    const void *ascales;    /* bf16 [K/64, M_pad] (INT4) or fp8-e4m3 [K/16, M_pad] (NVFP4)          */
+    const void *ascales;    /* as written by operator 1: bf16 [K/64][M_pad] or fp8 [K/64][M_pad][4] */
     const void *wgt;        /* native qweight (svdq_repack_qweight)                                 */
     const void *wscales;    /* native fp16 scales (svdq_repack_wscales / _wmscales)                 */
     const float *colnorm;   /* fp32 [N] from the same repack call                                   */
@@ -118,7 +120,7 @@ typedef struct svdq_gemm_args {
     void *out;              /* bf16 [M_out, N_out] row-major, or NULL                               */
     /* next-layer fusion (all NULL unless qout is given) */
     void *qout;             /* u8 native activation tiles [M_pad, N/2] for the next layer           */
-    void *oscales;          /* bf16 [N/64, M_pad] (INT4 unsigned) or fp8 [N/16, M_pad] (NVFP4)      */
+    void *oscales;          /* bf16 [N/64][M_pad] (INT4 unsigned) or fp8 [N/64][M_pad][4] (NVFP4)   */
     const float *next_smooth_rcp; /* fp32 [N] from svdq_repack_smooth of the next layer             */
     const void *next_lora_down;   /* native proj_down of the next layer ([N, R_down]) or NULL       */
     float *next_lora_act_out;     /* fp32 [M_pad, R_down]; zeroed and accumulated by the call       */

@@ -38,8 +38,10 @@ namespace {
 
 constexpr int BM = 256, BN = 256;
 constexpr int STAGES = 4;
-constexpr int STAGE_A = 0, STAGE_B = 8192, STAGE_AS = 16384, STAGE_BS = 16384 + 2048;
-constexpr int STAGE_BYTES = 16384 + 4096;  // 8 KB A codes, 8 KB B codes, 2 KB + 2 KB packed scales
+// per stage: 8 KB A codes, 8 KB B codes, then 16 bytes of packed fp16 scale pairs per row / column:
+// INT4 {s,s} {s/16,s/16} (8 bytes used); NVFP4 one {s,s} pair for each of the four 16-groups
+constexpr int STAGE_A = 0, STAGE_B = 8192, STAGE_AS = 16384, STAGE_BS = 16384 + 4096;
+constexpr int STAGE_BYTES = 16384 + 8192;
 constexpr int OUT_LD = 136;                // bf16 elements per row of the store-staging slab (128 + pad)
 constexpr int ROWNORM_OFF = STAGES * STAGE_BYTES;  // fp32 [256] row de-normalisation factors
 constexpr int ROWMAX_OFF = ROWNORM_OFF + 1024;     // u32 [256] scratch for the row maximum
@@ -101,6 +103,21 @@ __device__ inline half8_t dequant_word(uint32_t w, half2_t s, half2_t s16, const
     return half8_t{a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
 }
 
+// 8 E2M1 patterns of one word -> 8 fp16 values pattern_value * scale, slot order [0..7].  The
+// hardware conversion yields the exact E2M1 value (its scale operand only contributes an exponent).
+__device__ inline half8_t dequant_word_fp4(uint32_t w, half2_t s) {
+    const half2_t t0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 0) * s;
+    const half2_t t1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 1) * s;
+    const half2_t t2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 2) * s;
+    const half2_t t3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 3) * s;
+    return half8_t{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+}
+
+__device__ inline float e4m3_to_f32(uint32_t b) {
+    const uint32_t ex = (b >> 3) & 0xF, m = b & 7;
+    return ex == 0 ? ldexpf((float)m, -9) : ldexpf((float)(8 + m), (int)ex - 10);
+}
+
 __global__ void zero_f32_kernel(float *p, int64_t n) {
     const int64_t i = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) * 4;
     if (i + 3 < n) *(float4_t *)(p + i) = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -116,9 +133,8 @@ __device__ inline float gelu_tanh(float x) {
     return x * (0.5f + 0.5f * t);
 }
 
-template <bool ACT_UNSIGNED>
-__global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
-    constexpr bool FP4 = false;
+template <bool ACT_UNSIGNED, bool FP4>
+__global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -146,9 +162,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
     SVDQ_STAMP(0);
 
     // ---- prologue: largest activation scale of each of my 256 rows -> power-of-two renormalisation
-    rowmax[tid] = 0;
-    __syncthreads();
-    {
+    int my_shift;  // thread tid owns row tid of the block when staging scales
+    if (!FP4) {
+        rowmax[tid] = 0;
+        __syncthreads();
         const int oct = tid & 31, gs = tid >> 5;
         uint32_t mx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (int g = gs; g < kgroups; g += 8) {
@@ -161,14 +178,23 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
         }
 #pragma unroll
         for (int j = 0; j < 8; j++) atomicMax(&rowmax[8 * oct + j], mx[j]);
-    }
-    __syncthreads();
-    int my_shift;  // thread tid owns row tid of the block when staging scales
-    {
+        __syncthreads();
         const int ex = (int)(rowmax[tid] >> 7);  // biased bf16 exponent of the row maximum
         my_shift = ex == 0 ? 0 : NORM_TARGET_EXP - (ex - 127);
-        rownorm[tid] = ldexpf(1.0f, -my_shift);
+    } else {
+        // NVFP4: four e4m3 scales per (row, 64-group) packed in one word; e4m3 patterns of
+        // non-negative values order like unsigned bytes
+        const uint32_t *sp = (const uint32_t *)p.ascales + m0 + tid;
+        uint32_t mx = 0;
+        for (int g = 0; g < kgroups; g++) {
+            const uint32_t v = sp[(size_t)g * p.M_pad];
+            mx = max(max(mx, v & 0x7Fu), max((v >> 8) & 0x7Fu, max((v >> 16) & 0x7Fu, (v >> 24) & 0x7Fu)));
+        }
+        int ex = 0;
+        if (mx) frexpf(e4m3_to_f32(mx), &ex);  // value in [2^(ex-1), 2^ex)
+        my_shift = mx == 0 ? 0 : NORM_TARGET_EXP - (ex - 1);
     }
+    rownorm[tid] = ldexpf(1.0f, -my_shift);
     const bool col_ok = n0 + tid < p.N;
     SVDQ_STAMP(1);
 
@@ -190,8 +216,11 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
         a_src[j] = p.act + (size_t)(mt0 + t) * kgroups * TILE_BYTES + lane * 16;
         b_src[j] = p.wgt + (size_t)tb * kgroups * TILE_BYTES + lane * 16;
     }
-    const uint16_t *as_src = p.ascales + m0 + tid;
-    const _Float16 *bs_src = p.wscales + (col_ok ? n0 + tid : p.N - 1);
+    // scale sources: INT4 one bf16 / fp16 value per (group, row / column); NVFP4 one word of four e4m3
+    // (activations) or four fp16 (weights) per (64-group, row / column)
+    const uint8_t *as_src = (const uint8_t *)p.ascales + (size_t)(m0 + tid) * (FP4 ? 4 : 2);
+    const uint8_t *bs_src = (const uint8_t *)p.wscales + (size_t)(col_ok ? n0 + tid : p.N - 1) * (FP4 ? 8 : 2);
+    const size_t as_stride = (size_t)p.M_pad * (FP4 ? 4 : 2), bs_stride = (size_t)p.N * (FP4 ? 8 : 2);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     auto issue_codes = [&](int g) {  // 4 vector-memory operations
         const int gc = g < kgroups ? g : kgroups - 1;  // surplus copies at the tail are never consumed
@@ -204,19 +233,39 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
                          :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(b_src[j] + (size_t)gc * TILE_BYTES) : "memory");
         }
     };
-    auto issue_scales = [&](int g, uint32_t &ra, uint32_t &rb) {  // 2 vector-memory operations
+    auto issue_scales = [&](int g, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
         const int gc = g < kgroups ? g : kgroups - 1;
-        asm volatile("global_load_ushort %0, %1, off" : "=v"(ra) : "v"(as_src + (size_t)gc * p.M_pad) : "memory");
-        asm volatile("global_load_ushort %0, %1, off" : "=v"(rb) : "v"(bs_src + (size_t)gc * p.N) : "memory");
+        if (!FP4) {
+            uint32_t t;
+            asm volatile("global_load_ushort %0, %1, off" : "=v"(ra) : "v"(as_src + gc * as_stride) : "memory");
+            asm volatile("global_load_ushort %0, %1, off" : "=v"(t) : "v"(bs_src + gc * bs_stride) : "memory");
+            rb[0] = t;
+        } else {
+            asm volatile("global_load_dword %0, %1, off" : "=v"(ra) : "v"(as_src + gc * as_stride) : "memory");
+            asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(rb) : "v"(bs_src + gc * bs_stride) : "memory");
+        }
     };
-    auto store_scales = [&](int g, uint32_t ra, uint32_t rb) {
+    auto store_scales = [&](int g, uint32_t ra, u32x2_t rb) {
         uint8_t *base = lds + (g % STAGES) * STAGE_BYTES;
-        const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), my_shift);
-        const _Float16 sb = col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb) : (_Float16)0.f;
-        const _Float16 sa16 = sa * (_Float16)0.0625f;
-        const _Float16 sb16 = sb * (_Float16)0.0625f;
-        *(u32x2_t *)(base + STAGE_AS + tid * 8) = u32x2_t{as_u32(half2_t{sa, sa}), as_u32(half2_t{sa16, sa16})};
-        *(u32x2_t *)(base + STAGE_BS + tid * 8) = u32x2_t{as_u32(half2_t{sb, sb}), as_u32(half2_t{sb16, sb16})};
+        if (!FP4) {
+            const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), my_shift);
+            const _Float16 sb = col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb[0]) : (_Float16)0.f;
+            const _Float16 sa16 = sa * (_Float16)0.0625f;
+            const _Float16 sb16 = sb * (_Float16)0.0625f;
+            *(u32x2_t *)(base + STAGE_AS + tid * 16) = u32x2_t{as_u32(half2_t{sa, sa}), as_u32(half2_t{sa16, sa16})};
+            *(u32x2_t *)(base + STAGE_BS + tid * 16) = u32x2_t{as_u32(half2_t{sb, sb}), as_u32(half2_t{sb16, sb16})};
+        } else {
+            u32x4_t pa, pb;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const _Float16 sa = (_Float16)ldexpf(e4m3_to_f32((ra >> (8 * j)) & 0x7Fu), my_shift);
+                pa[j] = as_u32(half2_t{sa, sa});
+                const uint32_t hb = col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
+                pb[j] = hb | (hb << 16);
+            }
+            *(u32x4_t *)(base + STAGE_AS + tid * 16) = pa;
+            *(u32x4_t *)(base + STAGE_BS + tid * 16) = pb;
+        }
     };
 
     float16_t acc[4][4];
@@ -228,9 +277,11 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     // prologue: scales of groups 0..2 and codes of groups 0..3
-    uint32_t sa_e, sb_e, sa_o, sb_o;  // scale registers in flight: even / odd groups
+    uint32_t sa_e, sa_o;  // scale registers in flight: even / odd groups
+    u32x2_t sb_e, sb_o;
     {
-        uint32_t s0a, s0b, s1a, s1b;
+        uint32_t s0a, s1a;
+        u32x2_t s0b, s1b;
         issue_scales(0, s0a, s0b);
         issue_scales(1, s1a, s1b);
         issue_scales(2, sa_e, sb_e);
@@ -269,14 +320,19 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
         for (int t = 0; t < 4; t++) {
             ar[t] = *(const u32x4_t *)(base + STAGE_A + (wm * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
             br[t] = *(const u32x4_t *)(base + STAGE_B + (wn * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
-            as[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 8);
-            bs[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 8);
+            as[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 16 + (FP4 ? h * 8 : 0));
+            bs[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 16 + (FP4 ? h * 8 : 0));
         }
     };
 #define SVDQ_CONVERT(AR, BR, AS, BS, I, A, B)                                                             \
     _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                       \
-        A[t] = dequant_word(AR[t][I], as_half2(AS[t][0]), as_half2(AS[t][1]), dc, dc.off1, dc.off16);       \
-        B[t] = dequant_word(BR[t][I], as_half2(BS[t][0]), as_half2(BS[t][1]), dc, dc.woff1, dc.woff16);              \
+        if (!FP4) {                                                                                       \
+            A[t] = dequant_word(AR[t][I], as_half2(AS[t][0]), as_half2(AS[t][1]), dc, dc.off1, dc.off16); \
+            B[t] = dequant_word(BR[t][I], as_half2(BS[t][0]), as_half2(BS[t][1]), dc, dc.woff1, dc.woff16); \
+        } else { /* word I of the lane's 32 codes lies in 16-group 2h + I/2 */                             \
+            A[t] = dequant_word_fp4(AR[t][I], as_half2(AS[t][(I) >> 1]));                                  \
+            B[t] = dequant_word_fp4(BR[t][I], as_half2(BS[t][(I) >> 1]));                                  \
+        }                                                                                                 \
     }
 #define SVDQ_MFMA(A, B)                                                                                   \
     _Pragma("unroll") for (int mt = 0; mt < 4; mt++) _Pragma("unroll") for (int nt = 0; nt < 4; nt++)     \
@@ -491,10 +547,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_int4_kernel(GemmParams p) {
                 } else {
                     uint32_t sc[2];
                     quantize_nvfp4_two_groups(y, words, sc);
-                    uint8_t *os = (uint8_t *)p.oscales;
-                    const int g16 = (wcol0 + qc * 32) / 16;
-                    os[(size_t)g16 * p.M_pad + m] = (uint8_t)sc[0];
-                    os[(size_t)(g16 + 1) * p.M_pad + m] = (uint8_t)sc[1];
+                    uint16_t *os = (uint16_t *)p.oscales;  // [N/64][M_pad][4]
+                    os[((size_t)gidx * p.M_pad + m) * 2 + (qc & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
                 }
                 *(u32x4_t *)(p.qout + ((size_t)(m / 32) * ngroups_out + gidx) * TILE_BYTES + (m % 32) * 32 + 16 * (qc & 1)) = words;
             }
@@ -531,7 +585,7 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
                   (uintptr_t)a->lora_up) % 16 == 0, "gemm: pointers must be 16-byte aligned");
     SVDQ_REQUIRE(a->M_pad * a->N < (1ll << 40) && a->K < (1 << 24), "gemm: shape too large");
     if (a->fuse_silu) return fail(SVDQ_EUNSUPPORTED, "gemm: fuse_silu is not implemented");
-    if (a->fp4) return fail(SVDQ_EUNSUPPORTED, "gemm: NVFP4 operands are not implemented yet");
+    if (a->fp4 && a->act_unsigned) return fail(SVDQ_EINVAL, "gemm: NVFP4 activations are never unsigned");
     if (a->qout) {
         SVDQ_REQUIRE(a->oscales && a->next_smooth_rcp, "gemm: qout needs oscales and next_smooth_rcp");
         SVDQ_REQUIRE(((uintptr_t)a->qout | (uintptr_t)a->next_smooth_rcp) % 16 == 0, "gemm: qout pointers must be 16-byte aligned");
@@ -574,7 +628,7 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
 #endif
 
     const int nwg = (int)(a->M_pad / BM) * (int)((a->N + BN - 1) / BN);
-    auto kern = a->act_unsigned ? gemm_w4a4_int4_kernel<true> : gemm_w4a4_int4_kernel<false>;
+    auto kern = a->fp4 ? gemm_w4a4_kernel<false, true> : a->act_unsigned ? gemm_w4a4_kernel<true, false> : gemm_w4a4_kernel<false, false>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
     if (p.next_lora_out) {  // the low-rank projection for the next layer is accumulated across column blocks

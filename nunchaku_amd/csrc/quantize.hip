@@ -115,9 +115,9 @@ __global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) 
             } else {
                 uint32_t sc[2];
                 quantize_nvfp4_two_groups(y, words, sc);
-                uint8_t *os = (uint8_t *)p.oscales;
-                os[(size_t)(8 * c + 2 * q) * p.M_pad + row] = (uint8_t)sc[0];
-                os[(size_t)(8 * c + 2 * q + 1) * p.M_pad + row] = (uint8_t)sc[1];
+                // NVFP4 scales: [K/64][M_pad][4] -- the four 16-groups of a 64-group side by side
+                uint16_t *os = (uint16_t *)p.oscales;
+                os[((size_t)(2 * c + (q >> 1)) * p.M_pad + row) * 2 + (q & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
             }
             *(u32x4_t *)dst = words;
         }

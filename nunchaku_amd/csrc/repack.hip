@@ -98,7 +98,7 @@ __global__ void repack_wmscales_kernel(const uint8_t *__restrict__ src, _Float16
     }
     for (int64_t g = 0; g < G; g++) {
         const int64_t s = (((bn * ktiles + g / 4) * 32 + lane) * 4 + p) * 4 + (g % 4);
-        dst[g * N + n] = (_Float16)ldexpf(e4m3_to_f32(src[s]), e);
+        dst[((g / 4) * N + n) * 4 + (g % 4)] = (_Float16)ldexpf(e4m3_to_f32(src[s]), e);  // [K/64][N][4]
     }
     colnorm[n] = ldexpf(1.0f, -e);
 }

@@ -39,8 +39,9 @@ def repack_qweight(qweight: torch.Tensor, fp4: bool = False) -> torch.Tensor:
 
 
 def repack_wscales(wscales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
-    """bf16 [K/64, N] (or fp8 [K/16, N]) reference order -> fp16 column-normalised scales of the same
-    shape; the fp32 per-column factor that undoes the normalisation rides along as ``.colnorm``."""
+    """bf16 [K/64, N] (or fp8 [K/16, N]) reference order -> fp16 column-normalised scales with the
+    same element count (INT4: ``[K/64][N]``; NVFP4: ``[K/64][N][4]`` viewed as ``[K/16, N]``); the
+    fp32 per-column factor that undoes the normalisation rides along as ``.colnorm``."""
     nv.require_gpu(wscales, "wscales")
     G, N = wscales.shape
     out = torch.empty(G, N, dtype=torch.float16, device=wscales.device)
@@ -133,6 +134,23 @@ def act_to_logical(act: torch.Tensor, K: int, fp4: bool = False, unsigned: bool 
     if not fp4 and not unsigned:
         codes = codes - 8
     return codes.to(torch.int8)
+
+
+def scales_to_logical(scales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
+    """Activation scales as the kernels store them -> ``[K/G, M_pad]`` group-major.  INT4 scales are
+    stored that way already; NVFP4 scales are stored ``[K/64][M_pad][4]``."""
+    if not fp4:
+        return scales
+    G16, M_pad = scales.shape
+    return scales.view(torch.uint8).reshape(G16 // 4, M_pad, 4).permute(0, 2, 1).reshape(G16, M_pad).contiguous().view(scales.dtype)
+
+
+def logical_to_scales(scales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
+    """Inverse of :func:`scales_to_logical`."""
+    if not fp4:
+        return scales
+    G16, M_pad = scales.shape
+    return scales.view(torch.uint8).reshape(G16 // 4, 4, M_pad).permute(0, 2, 1).contiguous().reshape(G16, M_pad).view(scales.dtype)
 
 
 def logical_to_act(codes: torch.Tensor, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:

@@ -20,7 +20,7 @@ def _run(dev, x, layer, fp4=False, smooth=True):
         x.to(dev), lora_down=sd["proj_down"].to(dev), smooth=sd["smooth_factor"].to(dev) if smooth else None, fp4=fp4
     )
     torch.cuda.synchronize()
-    return packing.act_to_logical(out.cpu(), x.shape[1], fp4=fp4), osc.cpu(), la.cpu()
+    return packing.act_to_logical(out.cpu(), x.shape[1], fp4=fp4), packing.scales_to_logical(osc.cpu(), fp4), la.cpu()
 
 
 def _check(x, layer, codes, osc, la, fp4=False, smooth=True):

@@ -63,7 +63,9 @@ def test_repack_micro_scales(dev):
     src = torch.from_numpy(z["mscales_packed"]).view(torch.float8_e4m3fn).to(dev)
     ws = packing.repack_wscales(src, fp4=True)
     logical = torch.from_numpy(z["mscales_logical"]).view(torch.float8_e4m3fn).float()
-    assert torch.equal(ws.float().cpu() * ws.colnorm.cpu()[None, :], logical)
+    G16, N = logical.shape
+    got = ws.float().cpu().reshape(G16 // 4, N, 4).permute(0, 2, 1).reshape(G16, N)  # [K/64][N][4] -> [K/16][N]
+    assert torch.equal(got * ws.colnorm.cpu()[None, :], logical)
 
 
 def test_repack_random_larger(dev):
