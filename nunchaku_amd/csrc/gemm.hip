@@ -13,17 +13,17 @@
 // definition up to fp32 summation order; no per-group post-scaling exists.
 //
 // Range: activation scales are renormalised per row and weight scales per column by powers of two
-// (largest scale of a row / column moved into [2^11, 2^12)), so the fp16 products never overflow and
+// (largest scale of a row / column moved into [2^10, 2^11)), so the fp16 products never overflow and
 // only contributions 2^-25 below the largest of their row / column can underflow.  The shifts are
 // undone exactly in the epilogue.
 //
-// Dequantization of one 32-bit word (8 codes, element e in bits [4e, 4e+4)):
-//   (w & 0x000F000F) | 0x64006400 -> two fp16 values 1024 + u          (elements 0 and 4)
-//   (w & 0x00F000F0) | 0x64006400 -> two fp16 values 1024 + 16 u       (elements 1 and 5)
-//   same on w >> 8                                                     (elements 2, 6 and 3, 7)
-// followed by a packed fp16 subtract of the bias (1032 / 1152 for offset-binary signed codes,
-// 1024 for unsigned ones) and a packed multiply by the scale (or scale / 16).  Both operands use
-// the same element-to-slot order, so the contraction pairs equal k.
+// Dequantization of one INT4 word (8 codes; the nibble word is stored rotated left by 2 bits so that
+// two codes sit on fp16 mantissa bits [9:6] of the two halves, the other pairs a shift / rotate away):
+//   (w' & 0x03C003C0) | 0x3C003C00 -> two fp16 values 1 + u/16,  w' in {w, w >> 4, w << 4, rotl(w, 8)}
+//   packed fma with (16 s, -24 s)   -> (u - 8) s, exact (offset-binary signed codes; -16 s: unsigned)
+// = 11 VALU instructions per 8 codes.  Both operands use the same element-to-slot order, so the
+// contraction pairs equal k.  NVFP4 words use the hardware E2M1 -> fp16 conversion and one packed
+// multiply per pair (8 instructions per 8 codes).
 //
 // Tiling: workgroup = 4 waves (2 x 2), block tile 256 x 256, wave tile 128 x 128 = 4 x 4 MFMA tiles,
 // 256 fp32 accumulators per lane.  Operand tiles are staged through a 3-deep LDS ring, one k-group
@@ -39,14 +39,15 @@ namespace {
 constexpr int BM = 256, BN = 256;
 constexpr int STAGES = 4;
 // per stage: 8 KB A codes, 8 KB B codes, then 16 bytes of packed fp16 scale pairs per row / column:
-// INT4 {s,s} {s/16,s/16} (8 bytes used); NVFP4 one {s,s} pair for each of the four 16-groups
+// INT4 {16s,16s} {-24s,-24s} (8 bytes used; -16s for unsigned codes); NVFP4 one {s,s} pair for each
+// of the four 16-groups
 constexpr int STAGE_A = 0, STAGE_B = 8192, STAGE_AS = 16384, STAGE_BS = 16384 + 4096;
 constexpr int STAGE_BYTES = 16384 + 8192;
 constexpr int OUT_LD = 136;                // bf16 elements per row of the store-staging slab (128 + pad)
 constexpr int ROWNORM_OFF = STAGES * STAGE_BYTES;  // fp32 [256] row de-normalisation factors
 constexpr int ROWMAX_OFF = ROWNORM_OFF + 1024;     // u32 [256] scratch for the row maximum
 constexpr int LDS_BYTES = ROWMAX_OFF + 1024;
-constexpr int NORM_TARGET_EXP = 11;
+constexpr int NORM_TARGET_EXP = 10;
 
 #ifdef SVDQ_GEMM_TIMING
 #define SVDQ_STAMP(i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 8 + (i)] = __builtin_readcyclecounter()
@@ -82,24 +83,23 @@ __device__ inline half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2
 __device__ inline uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
 
 struct DequantConsts {
-    uint32_t magic;   // fp16 pair 1024.0: OR-ing a 4-bit code into its low mantissa bits gives 1024 + u
-    uint32_t mask0, mask4;  // 0x000F000F / 0x00F000F0, kept opaque so that (w & mask) | magic becomes one v_and_or_b32
-    half2_t off1;     // 1024 + 8 (offset-binary signed code in bits 0..3) or 1024 (unsigned)
-    half2_t off16;    // 1024 + 128 (code in bits 4..7) or 1024
-    half2_t woff1, woff16;  // the same for the weight operand (always offset-binary)
+    uint32_t magic;  // fp16 pair 1.0: OR-ing a code into mantissa bits [9:6] gives 1 + u/16
+    uint32_t mask;   // 0x03C003C0; kept opaque so that (w & mask) | magic becomes one v_and_or_b32
 };
 
-// 8 codes of one word -> 8 fp16 values (code - bias) * scale in slot order [0,4,1,5,2,6,3,7]
-__device__ inline half8_t dequant_word(uint32_t w, half2_t s, half2_t s16, const DequantConsts &dc, half2_t off1, half2_t off16) {
-    const uint32_t w8 = w >> 8;
-    const half2_t t0 = as_half2((w & dc.mask0) | dc.magic);
-    const half2_t t1 = as_half2((w & dc.mask4) | dc.magic);
-    const half2_t t2 = as_half2((w8 & dc.mask0) | dc.magic);
-    const half2_t t3 = as_half2((w8 & dc.mask4) | dc.magic);
-    const half2_t a0 = (t0 - off1) * s;
-    const half2_t a1 = (t1 - off16) * s16;
-    const half2_t a2 = (t2 - off1) * s;
-    const half2_t a3 = (t3 - off16) * s16;
+// 8 INT4 codes of one (rotated) word -> 8 fp16 values (code - bias) * scale.  `mul` = 16 * scale and
+// `add` = -(16 + bias) * scale as fp16 pairs (bias 8 for offset-binary signed codes, 0 for unsigned):
+// fma(1 + u/16, 16 s, -(16 + bias) s) = (u - bias) s with a single, exact rounding.
+// Slot order (identical for both operands): elements [1,5,2,6,0,4,7,3].
+__device__ inline half8_t dequant_word(uint32_t w, half2_t mul, half2_t add, const DequantConsts &dc) {
+    const half2_t t0 = as_half2((w & dc.mask) | dc.magic);
+    const half2_t t1 = as_half2(((w >> 4) & dc.mask) | dc.magic);
+    const half2_t t2 = as_half2(((w << 4) & dc.mask) | dc.magic);
+    const half2_t t3 = as_half2((__builtin_amdgcn_alignbit(w, w, 24) & dc.mask) | dc.magic);
+    const half2_t a0 = __builtin_elementwise_fma(t0, mul, add);
+    const half2_t a1 = __builtin_elementwise_fma(t1, mul, add);
+    const half2_t a2 = __builtin_elementwise_fma(t2, mul, add);
+    const half2_t a3 = __builtin_elementwise_fma(t3, mul, add);
     return half8_t{a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
 }
 
@@ -250,10 +250,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         if (!FP4) {
             const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), my_shift);
             const _Float16 sb = col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb[0]) : (_Float16)0.f;
-            const _Float16 sa16 = sa * (_Float16)0.0625f;
-            const _Float16 sb16 = sb * (_Float16)0.0625f;
-            *(u32x2_t *)(base + STAGE_AS + tid * 16) = u32x2_t{as_u32(half2_t{sa, sa}), as_u32(half2_t{sa16, sa16})};
-            *(u32x2_t *)(base + STAGE_BS + tid * 16) = u32x2_t{as_u32(half2_t{sb, sb}), as_u32(half2_t{sb16, sb16})};
+            const _Float16 ma = sa * (_Float16)16.f, mb = sb * (_Float16)16.f;
+            const _Float16 na = sa * (_Float16)(ACT_UNSIGNED ? -16.f : -24.f), nb = sb * (_Float16)-24.f;
+            *(u32x2_t *)(base + STAGE_AS + tid * 16) = u32x2_t{as_u32(half2_t{ma, ma}), as_u32(half2_t{na, na})};
+            *(u32x2_t *)(base + STAGE_BS + tid * 16) = u32x2_t{as_u32(half2_t{mb, mb}), as_u32(half2_t{nb, nb})};
         } else {
             u32x4_t pa, pb;
 #pragma unroll
@@ -296,17 +296,12 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     __syncthreads();
     SVDQ_STAMP(2);
 
-    // conversion constants, pinned in vector registers (VOP3 cannot take literals, and a scalar
-    // operand on the packed instructions costs a wait state each time)
+    // conversion constants, pinned in registers (VOP3 cannot take literals; opaque values let the
+    // compiler form v_and_or_b32)
     DequantConsts dc;
-    dc.magic = 0x64006400u;
-    dc.off1 = ACT_UNSIGNED ? half2_t{(_Float16)1024.f, (_Float16)1024.f} : half2_t{(_Float16)1032.f, (_Float16)1032.f};
-    dc.off16 = ACT_UNSIGNED ? half2_t{(_Float16)1024.f, (_Float16)1024.f} : half2_t{(_Float16)1152.f, (_Float16)1152.f};
-    dc.woff1 = half2_t{(_Float16)1032.f, (_Float16)1032.f};
-    dc.woff16 = half2_t{(_Float16)1152.f, (_Float16)1152.f};
-    dc.mask0 = 0x000F000Fu;
-    dc.mask4 = 0x00F000F0u;
-    asm volatile("" : "+v"(dc.magic), "+v"(dc.off1), "+v"(dc.off16), "+v"(dc.woff1), "+v"(dc.woff16), "+s"(dc.mask0), "+s"(dc.mask4));
+    dc.magic = 0x3C003C00u;
+    dc.mask = 0x03C003C0u;
+    asm volatile("" : "+v"(dc.magic), "+s"(dc.mask));
 
     // Software pipeline over the 16-wide MFMA steps (4 per k-group): while the 16 MFMAs of a step run,
     // the VALU dequantizes the operands of the next step, so a wave never waits on its own
@@ -327,8 +322,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #define SVDQ_CONVERT(AR, BR, AS, BS, I, A, B)                                                             \
     _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                       \
         if (!FP4) {                                                                                       \
-            A[t] = dequant_word(AR[t][I], as_half2(AS[t][0]), as_half2(AS[t][1]), dc, dc.off1, dc.off16); \
-            B[t] = dequant_word(BR[t][I], as_half2(BS[t][0]), as_half2(BS[t][1]), dc, dc.woff1, dc.woff16); \
+            A[t] = dequant_word(AR[t][I], as_half2(AS[t][0]), as_half2(AS[t][1]), dc);                     \
+            B[t] = dequant_word(BR[t][I], as_half2(BS[t][0]), as_half2(BS[t][1]), dc);                     \
         } else { /* word I of the lane's 32 codes lies in 16-group 2h + I/2 */                             \
             A[t] = dequant_word_fp4(AR[t][I], as_half2(AS[t][(I) >> 1]));                                  \
             B[t] = dequant_word_fp4(BR[t][I], as_half2(BS[t][(I) >> 1]));                                  \
@@ -357,7 +352,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         /* an MFMA takes two issue slots, every other instruction one; 8 passes cover six of them */      \
         _Pragma("unroll") for (int k = 0; k < 32; k++) {                                                  \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
-            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);                                            \
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
             __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
         }                                                                                                 \

@@ -13,9 +13,10 @@ namespace {
 // Reference storage (packer.py:210-239, loader gemm_base.cuh:278-294): u32 words
 // [N/128][K/64][j:8][lane:32][c:4]; word c of lane (g = lane/4, t = lane%4) in 16-row tile j holds
 // row 16j + g + 8*(c>=2), columns 32*(c odd) + 8t + [0..8), element e in bits [4e, 4e+4).
-// Native: [N/32][K/64][32 rows][8 words], word w of a row holds columns 8w + [0..8).
+// Native: [N/32][K/64][32 rows][8 words], word w of a row holds columns 8w + [0..8); INT4 words are
+// made offset-binary and rotated (svdq_common.h).
 __global__ void repack_qweight_kernel(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, int64_t N, int64_t K,
-                                      uint32_t xor_mask) {
+                                      uint32_t xor_mask, int rot) {
     const int64_t total = N * K / 8;
     const int64_t kgroups = K / 64;
     for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
@@ -30,7 +31,8 @@ __global__ void repack_qweight_kernel(const uint32_t *__restrict__ src, uint32_t
         const int codd = w / 4, t = w % 4;
         const int lane = gl * 4 + t, c = chi * 2 + codd;
         const int64_t s = (((bn * kgroups + g) * 8 + j) * 32 + lane) * 4 + c;
-        dst[i] = src[s] ^ xor_mask;
+        const uint32_t word = src[s] ^ xor_mask;
+        dst[i] = rot ? rotl32(word, rot) : word;
     }
 }
 
@@ -44,8 +46,9 @@ __device__ inline int64_t wscale_src_index(int64_t g, int64_t n, int64_t G) {
     return ((bn * G + g) * 32 + (4 * a + c)) * 4 + (2 * b + d);
 }
 
-// exponent shift that puts the largest scale of a column into [2^11, 2^12)
-constexpr int NORM_TARGET_EXP = 11;
+// exponent shift that puts the largest scale of a column into [2^10, 2^11): 16 * scale and 24 * scale
+// (the packed-fma constants of the GEMM) then stay below the fp16 maximum
+constexpr int NORM_TARGET_EXP = 10;
 
 __global__ void repack_wscales_kernel(const uint16_t *__restrict__ src, _Float16 *__restrict__ dst,
                                       float *__restrict__ colnorm, int64_t N, int64_t G) {
@@ -171,7 +174,7 @@ int svdq_repack_qweight(const void *src, void *dst, int64_t N, int64_t K, int fp
     unsigned grid = blocks_for(total);
     if (grid > 65536u) grid = 65536u;
     hipLaunchKernelGGL(repack_qweight_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
-                       (uint32_t *)dst, N, K, fp4 ? 0u : 0x88888888u);
+                       (uint32_t *)dst, N, K, fp4 ? 0u : 0x88888888u, fp4 ? 0 : INT4_WORD_ROT);
     return check_launch("repack_qweight");
 }
 

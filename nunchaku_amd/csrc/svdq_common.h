@@ -66,9 +66,18 @@ __host__ __device__ inline uint32_t f32_to_bf16_bits(float f) {
 }
 
 // Native tile geometry of 4-bit operands (activations and weights alike):
-//   [rows/32][K/64][32 rows][32 bytes], byte b of a (row, 64-group) = elements 2b | (2b+1) << 4.
+//   [rows/32][K/64][32 rows][8 words]; word w of a (row, 64-group) holds elements 8w .. 8w+7.
+//   NVFP4: element e of a word in bits [4e, 4e+4) (plain nibbles).
+//   INT4 : the same nibble word rotated left by 2 bits (INT4_WORD_ROT), signed codes offset-binary
+//          (code + 8).  The rotation puts elements 1 and 5 on bits [9:6] / [25:22], i.e. onto the top
+//          mantissa bits of an fp16 pair, and every other pair one shift or rotate away from there:
+//          OR-ing 0x3C00 gives the fp16 value 1 + u/16, and one packed fma with (16 s, -24 s) yields
+//          (u - 8) s exactly.
 constexpr int TILE_ROWS = 32;
 constexpr int GROUP_K = 64;
 constexpr int TILE_BYTES = TILE_ROWS * GROUP_K / 2;  // 1024
+constexpr int INT4_WORD_ROT = 2;
+
+__host__ __device__ inline uint32_t rotl32(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
 
 }  // namespace svdq

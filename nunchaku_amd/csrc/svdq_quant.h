@@ -62,7 +62,8 @@ __device__ inline uint32_t f32_to_e2m1(float v) {
 
 // One lane holds 32 consecutive elements of a row = half of a 64-group; the other half lives in the
 // lane `partner_xor` away.  Produces the 16 bytes of codes of this half and the group scale.
-// Signed codes are emitted offset-binary (code + 8), unsigned ones as they are.
+// Signed codes are emitted offset-binary (code + 8), unsigned ones as they are; words are in the
+// rotated INT4 word format of svdq_common.h.
 template <bool UNSIGNED>
 __device__ inline void quantize_int4_half_group(const float (&y)[32], int partner_xor, u32x4_t &words, float &scale) {
     float amax = 0.f;
@@ -82,7 +83,7 @@ __device__ inline void quantize_int4_half_group(const float (&y)[32], int partne
             t = fminf(fmaxf(t, lo), hi);
             v[j] = __fadd_rn(t, magic);  // the rounded code sits in the low nibble of the bit pattern
         }
-        words[wi] = pack8(v);
+        words[wi] = rotl32(pack8(v), INT4_WORD_ROT);
     }
     scale = s;
 }

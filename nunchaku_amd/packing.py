@@ -120,20 +120,40 @@ def native(t: torch.Tensor | None, kind: str, fp4: bool = False) -> torch.Tensor
 
 
 # ---------------------------------------------------------------------------------------------
-# logical views of the kernels' private activation layout (for tests and debugging)
+# logical views of the kernels' private 4-bit tile layout (for tests and debugging)
 # ---------------------------------------------------------------------------------------------
 
 
+INT4_WORD_ROT = 2  # INT4 code words are stored rotated left by this many bits (csrc/svdq_common.h)
+
+
 def act_to_logical(act: torch.Tensor, K: int, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:
-    """Native activation tiles u8 [M_pad, K/2] ([M_pad/32][K/64][32][32 B]) -> one code per element,
-    int8 [M_pad, K] in row/column order.  INT4 signed codes are stored offset-binary (code + 8)."""
+    """Native activation tiles u8 [M_pad, K/2] ([M_pad/32][K/64][32 rows][8 words]) -> one code per
+    element, int8 [M_pad, K] in row/column order.  INT4 words are stored rotated left by 2 bits and
+    signed codes offset-binary (code + 8); NVFP4 words are plain nibbles."""
     M_pad = act.shape[0]
-    t = act.reshape(M_pad // 32, K // 64, 32, 32).permute(0, 2, 1, 3).reshape(M_pad, K // 2).to(torch.int16)
-    lo, hi = t & 0xF, (t >> 4) & 0xF
-    codes = torch.stack([lo, hi], dim=-1).reshape(M_pad, K)
+    w = act.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    if not fp4:
+        w = ((w >> INT4_WORD_ROT) | (w << (32 - INT4_WORD_ROT))) & 0xFFFFFFFF
+    nib = torch.stack([(w >> (4 * e)) & 0xF for e in range(8)], dim=-1)  # [M_pad, K/8, 8] in tile order
+    codes = nib.reshape(M_pad // 32, K // 64, 32, 64).permute(0, 2, 1, 3).reshape(M_pad, K)
     if not fp4 and not unsigned:
         codes = codes - 8
     return codes.to(torch.int8)
+
+
+def logical_to_act(codes: torch.Tensor, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:
+    """Inverse of :func:`act_to_logical` (used by tests to feed hand-made codes to the GEMM)."""
+    M_pad, K = codes.shape
+    c = codes.to(torch.int64)
+    if not fp4 and not unsigned:
+        c = c + 8
+    c = (c & 0xF).reshape(M_pad // 32, 32, K // 64, 8, 8).permute(0, 2, 1, 3, 4)  # tile, group, row, word, element
+    w = sum(c[..., e] << (4 * e) for e in range(8))
+    if not fp4:
+        w = ((w << INT4_WORD_ROT) | (w >> (32 - INT4_WORD_ROT))) & 0xFFFFFFFF
+    w = torch.where(w >= 2**31, w - 2**32, w).to(torch.int32)
+    return w.contiguous().view(torch.uint8).reshape(M_pad, K // 2)
 
 
 def scales_to_logical(scales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
@@ -151,14 +171,3 @@ def logical_to_scales(scales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
         return scales
     G16, M_pad = scales.shape
     return scales.view(torch.uint8).reshape(G16 // 4, 4, M_pad).permute(0, 2, 1).contiguous().reshape(G16, M_pad).view(scales.dtype)
-
-
-def logical_to_act(codes: torch.Tensor, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:
-    """Inverse of :func:`act_to_logical` (used by tests to feed hand-made codes to the GEMM)."""
-    M_pad, K = codes.shape
-    c = codes.to(torch.int16)
-    if not fp4 and not unsigned:
-        c = c + 8
-    c = c & 0xF
-    packed = (c[:, 0::2] | (c[:, 1::2] << 4)).to(torch.uint8)
-    return packed.reshape(M_pad // 32, 32, K // 64, 32).permute(0, 2, 1, 3).contiguous().reshape(M_pad, K // 2)
