@@ -62,17 +62,38 @@ class GemmArgs(ctypes.Structure):
     ]
 
 
-def build(verbose: bool = False) -> Path:
+GEMM_VARIANTS = 6  # gemm_variant.hip is compiled once per kernel variant (-DSVDQ_VARIANT=n)
+
+
+def build(verbose: bool = False, extra_flags: tuple[str, ...] = (), lib_path: Path | None = None) -> Path:
     """Compile the HIP sources for gfx950 into ``libsvdq_amd.so`` next to this file (hipcc
-    cross-compiles; no GPU is needed)."""
+    cross-compiles; no GPU is needed).  Translation units are compiled in parallel, then linked."""
+    import concurrent.futures
+    import tempfile
+
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, *[str(_CSRC / s) for s in SOURCES], "-o", str(LIB_PATH)]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + res.stderr[-4000:])
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"] + list(extra_flags)
+    out = Path(lib_path) if lib_path else LIB_PATH
+    with tempfile.TemporaryDirectory(prefix="svdq_build_") as tmp:
+        jobs = [([str(_CSRC / src)], Path(tmp) / (src + ".o")) for src in SOURCES]
+        jobs += [([str(_CSRC / "gemm_variant.hip"), f"-DSVDQ_VARIANT={v}"], Path(tmp) / f"gemm_variant_{v}.o") for v in range(GEMM_VARIANTS)]
+
+        def compile_one(job):
+            args, obj = job
+            return subprocess.run([hipcc, *flags, "-c", *args, "-o", str(obj)], capture_output=True, text=True)
+
+        with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+            results = list(pool.map(compile_one, jobs))
+        for (args, _), res in zip(jobs, results):
+            if res.returncode != 0:
+                raise RuntimeError(f"hipcc failed on {args}:\n" + res.stderr[-4000:])
+        link = subprocess.run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *[str(o) for _, o in jobs], "-o", str(out)],
+                              capture_output=True, text=True)
+        if link.returncode != 0:
+            raise RuntimeError("hipcc link failed:\n" + link.stderr[-4000:])
     if verbose:
-        print(" ".join(cmd))
-    return LIB_PATH
+        print(f"built {out}")
+    return out
 
 
 _lib = None

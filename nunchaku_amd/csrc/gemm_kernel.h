@@ -1,0 +1,541 @@
+// Operator 2: W4A4 GEMM with fused epilogue for gfx950.  Counterpart of gemm_w4a4_kernel /
+// gemm_w4a4_fp4_kernel (src/kernels/zgemm/gemm_w4a4.cuh:1046-1095, :358-405) and of the epilogue
+// chain composed in gemm_w4a4_launch_impl.cuh:172-309.
+//
+// How the contraction is mapped to the matrix cores
+// -------------------------------------------------
+// Every 64-wide (16-wide for NVFP4) k-group carries its own activation scale (per row) and weight
+// scale (per column).  Applying them after an integer MFMA costs three VALU instructions per
+// accumulator per group, which caps an int8-MFMA kernel far below the matrix-core rate.  Instead
+// both operands are dequantized *in registers* to fp16 -- (code) * (scale) is exact in fp16 because
+// a 4-bit code has at most 3 significant bits and a bf16 / e4m3 scale at most 8 -- and fed to
+// v_mfma_f32_32x32x16_f16 with fp32 accumulation.  The result equals the fp32 dequantize-then-matmul
+// definition up to fp32 summation order; no per-group post-scaling exists.
+//
+// Range: activation scales are renormalised per row and weight scales per column by powers of two
+// (largest scale of a row / column moved into [2^10, 2^11)), so the fp16 products never overflow and
+// only contributions 2^-25 below the largest of their row / column can underflow.  The shifts are
+// undone exactly in the epilogue.
+//
+// Dequantization of one INT4 word (8 codes; the nibble word is stored rotated left by 2 bits so that
+// two codes sit on fp16 mantissa bits [9:6] of the two halves, the other pairs a shift / rotate away):
+//   (w' & 0x03C003C0) | 0x3C003C00 -> two fp16 values 1 + u/16,  w' in {w, w >> 4, w << 4, rotl(w, 8)}
+//   packed fma with (16 s, -24 s)   -> (u - 8) s, exact (offset-binary signed codes; -16 s: unsigned)
+// = 11 VALU instructions per 8 codes.  Both operands use the same element-to-slot order, so the
+// contraction pairs equal k.  NVFP4 words use the hardware E2M1 -> fp16 conversion and one packed
+// multiply per pair (8 instructions per 8 codes).
+//
+// Tiling: workgroup = 4 waves (2 x 2), block tile 256 x 256, wave tile 128 x 128 = 4 x 4 MFMA tiles,
+// 256 fp32 accumulators per lane.  Operand tiles are staged through a 3-deep LDS ring, one k-group
+// per stage; global loads for group g+3 are issued before the math of group g.
+#pragma once
+
+#include <type_traits>
+
+#include "gemm_params.h"
+#include "svdq_quant.h"
+
+namespace svdq {
+
+#ifdef SVDQ_GEMM_TIMING
+#define SVDQ_STAMP(i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 8 + (i)] = __builtin_readcyclecounter()
+#else
+#define SVDQ_STAMP(i)
+#endif
+
+
+
+__device__ inline half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ inline uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+
+struct DequantConsts {
+    uint32_t magic;  // fp16 pair 1.0: OR-ing a code into mantissa bits [9:6] gives 1 + u/16
+    uint32_t mask;   // 0x03C003C0; kept opaque so that (w & mask) | magic becomes one v_and_or_b32
+};
+
+// 8 INT4 codes of one (rotated) word -> 8 fp16 values (code - bias) * scale.  `mul` = 16 * scale and
+// `add` = -(16 + bias) * scale as fp16 pairs (bias 8 for offset-binary signed codes, 0 for unsigned):
+// fma(1 + u/16, 16 s, -(16 + bias) s) = (u - bias) s with a single, exact rounding.
+// Slot order (identical for both operands): elements [1,5,2,6,0,4,7,3].
+__device__ inline half8_t dequant_word(uint32_t w, half2_t mul, half2_t add, const DequantConsts &dc) {
+    const half2_t t0 = as_half2((w & dc.mask) | dc.magic);
+    const half2_t t1 = as_half2(((w >> 4) & dc.mask) | dc.magic);
+    const half2_t t2 = as_half2(((w << 4) & dc.mask) | dc.magic);
+    const half2_t t3 = as_half2((__builtin_amdgcn_alignbit(w, w, 24) & dc.mask) | dc.magic);
+    const half2_t a0 = __builtin_elementwise_fma(t0, mul, add);
+    const half2_t a1 = __builtin_elementwise_fma(t1, mul, add);
+    const half2_t a2 = __builtin_elementwise_fma(t2, mul, add);
+    const half2_t a3 = __builtin_elementwise_fma(t3, mul, add);
+    return half8_t{a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
+}
+
+// 8 E2M1 patterns of one word -> 8 fp16 values pattern_value * scale, slot order [0..7].  The
+// hardware conversion yields the exact E2M1 value (its scale operand only contributes an exponent).
+__device__ inline half8_t dequant_word_fp4(uint32_t w, half2_t s) {
+    const half2_t t0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 0) * s;
+    const half2_t t1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 1) * s;
+    const half2_t t2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 2) * s;
+    const half2_t t3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 3) * s;
+    return half8_t{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+}
+
+__device__ inline float e4m3_to_f32(uint32_t b) {
+    const uint32_t ex = (b >> 3) & 0xF, m = b & 7;
+    return ex == 0 ? ldexpf((float)m, -9) : ldexpf((float)(8 + m), (int)ex - 10);
+}
+
+__device__ inline float gelu_tanh(float x) {
+    // x * (0.5 + 0.5 * tanh(0.79788456 * (x + 0.044715 x^3)))   (epilogues.cuh:22-44)
+    const float u = 0.79788456f * (x + 0.044715f * x * x * x);
+    // tanh(u) = 1 - 2 / (exp(2u) + 1); exact enough in fp32 and safe for large |u|
+    const float e = __expf(2.0f * u);
+    const float t = 1.0f - 2.0f / (e + 1.0f);
+    return x * (0.5f + 0.5f * t);
+}
+
+// NEXT: the epilogue also prepares the next layer's input (GELU, quantize, low-rank down); the plain
+// variant carries none of that code or of its registers.
+template <bool ACT_UNSIGNED, bool FP4, bool NEXT>
+__global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r32 = lane & 31, h = lane >> 5;
+
+    // ---- block coordinates: consecutive ids of one XCD (id % 8) walk down M inside a band of N
+    const int mblocks = p.M_pad / BM, nblocks = (p.N + BN - 1) / BN;
+    const int nwg = mblocks * nblocks;
+    int id = blockIdx.x;
+    {
+        const int per_xcd = (nwg + 7) / 8;
+        const int xcd = id % 8, slot = id / 8;
+        const int lin = xcd * per_xcd + slot;
+        // when nwg is not a multiple of 8 some (xcd, slot) pairs fall outside: fall back to identity
+        id = (nwg % 8 == 0) ? lin : id;
+    }
+    const int bm = id % mblocks, bn = id / mblocks;
+    const int m0 = bm * BM, n0 = bn * BN;
+    const int kgroups = p.K / 64;
+    const int ntiles_total = p.N / 32;
+
+    float *rownorm = (float *)(lds + ROWNORM_OFF);
+    uint32_t *rowmax = (uint32_t *)(lds + ROWMAX_OFF);
+    SVDQ_STAMP(0);
+
+    // ---- prologue: largest activation scale of each of my 256 rows -> power-of-two renormalisation
+    int my_shift;  // thread tid owns row tid of the block when staging scales
+    if (!FP4) {
+        rowmax[tid] = 0;
+        __syncthreads();
+        const int oct = tid & 31, gs = tid >> 5;
+        uint32_t mx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int g = gs; g < kgroups; g += 8) {
+            const u32x4_t v = *(const u32x4_t *)(p.ascales + (size_t)g * p.M_pad + m0 + 8 * oct);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                mx[2 * j] = max(mx[2 * j], v[j] & 0x7FFFu);
+                mx[2 * j + 1] = max(mx[2 * j + 1], (v[j] >> 16) & 0x7FFFu);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) atomicMax(&rowmax[8 * oct + j], mx[j]);
+        __syncthreads();
+        const int ex = (int)(rowmax[tid] >> 7);  // biased bf16 exponent of the row maximum
+        my_shift = ex == 0 ? 0 : NORM_TARGET_EXP - (ex - 127);
+    } else {
+        // NVFP4: four e4m3 scales per (row, 64-group) packed in one word; e4m3 patterns of
+        // non-negative values order like unsigned bytes
+        const uint32_t *sp = (const uint32_t *)p.ascales + m0 + tid;
+        uint32_t mx = 0;
+        for (int g = 0; g < kgroups; g++) {
+            const uint32_t v = sp[(size_t)g * p.M_pad];
+            mx = max(max(mx, v & 0x7Fu), max((v >> 8) & 0x7Fu, max((v >> 16) & 0x7Fu, (v >> 24) & 0x7Fu)));
+        }
+        int ex = 0;
+        if (mx) frexpf(e4m3_to_f32(mx), &ex);  // value in [2^(ex-1), 2^ex)
+        my_shift = mx == 0 ? 0 : NORM_TARGET_EXP - (ex - 1);
+    }
+    rownorm[tid] = ldexpf(1.0f, -my_shift);
+    const bool col_ok = n0 + tid < p.N;
+    SVDQ_STAMP(1);
+
+    // ---- staging -----------------------------------------------------------------------------
+    // Code tiles go global -> LDS with asynchronous 16-byte copies (no registers, no ds_write);
+    // the two scale values per thread travel through registers because they are renormalised on the
+    // way.  All vector-memory traffic of the main loop is issued from volatile asm, in a fixed
+    // order and with a fixed count per iteration, so that one hand-placed s_waitcnt vmcnt(N) per
+    // iteration is exact: group g+4's codes and group g+3's scales are issued at the top of
+    // iteration g; the end of iteration g waits for group g+2 (ten newer operations may stay in
+    // flight), which iteration g+1 reads.  That leaves three iterations for a copy to land.
+    const int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mt0 = m0 / 32, nt0 = n0 / 32;
+    const uint8_t *a_src[2], *b_src[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int t = ca + 4 * j;
+        const int tb = nt0 + t < ntiles_total ? nt0 + t : ntiles_total - 1;  // clamped: its scales are zero
+        a_src[j] = p.act + (size_t)(mt0 + t) * kgroups * TILE_BYTES + lane * 16;
+        b_src[j] = p.wgt + (size_t)tb * kgroups * TILE_BYTES + lane * 16;
+    }
+    // scale sources: INT4 one bf16 / fp16 value per (group, row / column); NVFP4 one word of four e4m3
+    // (activations) or four fp16 (weights) per (64-group, row / column)
+    const uint8_t *as_src = (const uint8_t *)p.ascales + (size_t)(m0 + tid) * (FP4 ? 4 : 2);
+    const uint8_t *bs_src = (const uint8_t *)p.wscales + (size_t)(col_ok ? n0 + tid : p.N - 1) * (FP4 ? 8 : 2);
+    const size_t as_stride = (size_t)p.M_pad * (FP4 ? 4 : 2), bs_stride = (size_t)p.N * (FP4 ? 8 : 2);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    auto issue_codes = [&](int g) {  // 4 vector-memory operations
+        const int gc = g < kgroups ? g : kgroups - 1;  // surplus copies at the tail are never consumed
+        const uint32_t dst = lds_base + (g % STAGES) * STAGE_BYTES + ca * TILE_BYTES;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :: "s"(dst + STAGE_A + 4 * j * TILE_BYTES), "v"(a_src[j] + (size_t)gc * TILE_BYTES) : "memory");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(b_src[j] + (size_t)gc * TILE_BYTES) : "memory");
+        }
+    };
+    auto issue_scales = [&](int g, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
+        const int gc = g < kgroups ? g : kgroups - 1;
+        if (!FP4) {
+            uint32_t t;
+            asm volatile("global_load_ushort %0, %1, off" : "=v"(ra) : "v"(as_src + gc * as_stride) : "memory");
+            asm volatile("global_load_ushort %0, %1, off" : "=v"(t) : "v"(bs_src + gc * bs_stride) : "memory");
+            rb[0] = t;
+        } else {
+            asm volatile("global_load_dword %0, %1, off" : "=v"(ra) : "v"(as_src + gc * as_stride) : "memory");
+            asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(rb) : "v"(bs_src + gc * bs_stride) : "memory");
+        }
+    };
+    auto store_scales = [&](int g, uint32_t ra, u32x2_t rb) {
+        uint8_t *base = lds + (g % STAGES) * STAGE_BYTES;
+        if (!FP4) {
+            const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), my_shift);
+            const _Float16 sb = col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb[0]) : (_Float16)0.f;
+            const _Float16 ma = sa * (_Float16)16.f, mb = sb * (_Float16)16.f;
+            const _Float16 na = sa * (_Float16)(ACT_UNSIGNED ? -16.f : -24.f), nb = sb * (_Float16)-24.f;
+            *(u32x2_t *)(base + STAGE_AS + tid * 16) = u32x2_t{as_u32(half2_t{ma, ma}), as_u32(half2_t{na, na})};
+            *(u32x2_t *)(base + STAGE_BS + tid * 16) = u32x2_t{as_u32(half2_t{mb, mb}), as_u32(half2_t{nb, nb})};
+        } else {
+            u32x4_t pa, pb;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const _Float16 sa = (_Float16)ldexpf(e4m3_to_f32((ra >> (8 * j)) & 0x7Fu), my_shift);
+                pa[j] = as_u32(half2_t{sa, sa});
+                const uint32_t hb = col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
+                pb[j] = hb | (hb << 16);
+            }
+            *(u32x4_t *)(base + STAGE_AS + tid * 16) = pa;
+            *(u32x4_t *)(base + STAGE_BS + tid * 16) = pb;
+        }
+    };
+
+    float16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    // prologue: scales of groups 0..2 and codes of groups 0..3
+    uint32_t sa_e, sa_o;  // scale registers in flight: even / odd groups
+    u32x2_t sb_e, sb_o;
+    {
+        uint32_t s0a, s1a;
+        u32x2_t s0b, s1b;
+        issue_scales(0, s0a, s0b);
+        issue_scales(1, s1a, s1b);
+        issue_scales(2, sa_e, sb_e);
+        issue_codes(0);
+        issue_codes(1);
+        issue_codes(2);
+        issue_codes(3);
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(s0a), "+v"(s0b), "+v"(s1a), "+v"(s1b), "+v"(sa_e), "+v"(sb_e) :: "memory");
+        store_scales(0, s0a, s0b);
+        store_scales(1, s1a, s1b);
+    }
+    __syncthreads();
+    SVDQ_STAMP(2);
+
+    // conversion constants, pinned in registers (VOP3 cannot take literals; opaque values let the
+    // compiler form v_and_or_b32)
+    DequantConsts dc;
+    dc.magic = 0x3C003C00u;
+    dc.mask = 0x03C003C0u;
+    asm volatile("" : "+v"(dc.magic), "+s"(dc.mask));
+
+    // Software pipeline over the 16-wide MFMA steps (4 per k-group): while the 16 MFMAs of a step run,
+    // the VALU dequantizes the operands of the next step, so a wave never waits on its own
+    // conversions.  raw_* hold the packed codes and scales of the current k-group, *_n of the next.
+    u32x4_t araw[4], braw[4], araw_n[4], braw_n[4];
+    u32x2_t asc[4], bsc[4], asc_n[4], bsc_n[4];
+    half8_t a0[4], b0[4], a1[4], b1[4];
+    auto read_raw = [&](int st, u32x4_t (&ar)[4], u32x4_t (&br)[4], u32x2_t (&as)[4], u32x2_t (&bs)[4]) {
+        const uint8_t *base = lds + st * STAGE_BYTES;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            ar[t] = *(const u32x4_t *)(base + STAGE_A + (wm * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
+            br[t] = *(const u32x4_t *)(base + STAGE_B + (wn * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
+            as[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 16 + (FP4 ? h * 8 : 0));
+            bs[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 16 + (FP4 ? h * 8 : 0));
+        }
+    };
+#define SVDQ_CONVERT(AR, BR, AS, BS, I, A, B)                                                             \
+    _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                       \
+        if (!FP4) {                                                                                       \
+            A[t] = dequant_word(AR[t][I], as_half2(AS[t][0]), as_half2(AS[t][1]), dc);                     \
+            B[t] = dequant_word(BR[t][I], as_half2(BS[t][0]), as_half2(BS[t][1]), dc);                     \
+        } else { /* word I of the lane's 32 codes lies in 16-group 2h + I/2 */                             \
+            A[t] = dequant_word_fp4(AR[t][I], as_half2(AS[t][(I) >> 1]));                                  \
+            B[t] = dequant_word_fp4(BR[t][I], as_half2(BS[t][(I) >> 1]));                                  \
+        }                                                                                                 \
+    }
+#define SVDQ_MFMA(A, B)                                                                                   \
+    _Pragma("unroll") for (int mt = 0; mt < 4; mt++) _Pragma("unroll") for (int nt = 0; nt < 4; nt++)     \
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[mt], B[nt], acc[mt][nt], 0, 0, 0);
+    // one k-group; S_USE holds the scales of group G+2 (issued one iteration ago), S_LOAD receives G+3's
+#define SVDQ_GROUP(G, SA_USE, SB_USE, SA_LOAD, SB_LOAD)                                                   \
+    {                                                                                                     \
+        issue_scales((G) + 3, SA_LOAD, SB_LOAD);                                                          \
+        issue_codes((G) + 4);                                                                             \
+        SVDQ_CONVERT(araw, braw, asc, bsc, 1, a1, b1)                                                     \
+        SVDQ_MFMA(a0, b0)                                                                                 \
+        SVDQ_CONVERT(araw, braw, asc, bsc, 2, a0, b0)                                                     \
+        SVDQ_MFMA(a1, b1)                                                                                 \
+        read_raw(((G) + 1) % STAGES, araw_n, braw_n, asc_n, bsc_n);                                       \
+        SVDQ_CONVERT(araw, braw, asc, bsc, 3, a1, b1)                                                     \
+        SVDQ_MFMA(a0, b0)                                                                                 \
+        SVDQ_CONVERT(araw_n, braw_n, asc_n, bsc_n, 0, a0, b0)                                             \
+        SVDQ_MFMA(a1, b1)                                                                                 \
+        _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                   \
+            araw[t] = araw_n[t]; braw[t] = braw_n[t]; asc[t] = asc_n[t]; bsc[t] = bsc_n[t];               \
+        }                                                                                                 \
+        /* an MFMA takes two issue slots, every other instruction one; 8 passes cover six of them */      \
+        _Pragma("unroll") for (int k = 0; k < 32; k++) {                                                  \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
+        }                                                                                                 \
+        asm volatile("s_waitcnt vmcnt(10)" : "+v"(SA_USE), "+v"(SB_USE) :: "memory");                     \
+        store_scales((G) + 2, SA_USE, SB_USE);                                                            \
+        __syncthreads();                                                                                  \
+    }
+
+    read_raw(0, araw, braw, asc, bsc);
+    SVDQ_CONVERT(araw, braw, asc, bsc, 0, a0, b0)
+    for (int g = 0; g < kgroups; g += 2) {  // K is a multiple of 128: an even number of groups
+        SVDQ_GROUP(g, sa_e, sb_e, sa_o, sb_o)
+        SVDQ_GROUP(g + 1, sa_o, sb_o, sa_e, sb_e)
+    }
+#undef SVDQ_GROUP
+#undef SVDQ_CONVERT
+#undef SVDQ_MFMA
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // pin the accumulators in the accumulation registers across the loop exit: without this the
+    // register allocator may place the 256 copies into ordinary registers inside the loop body
+    asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]),
+                      "+a"(acc[1][2]), "+a"(acc[1][3]), "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]),
+                      "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
+    __syncthreads();
+    SVDQ_STAMP(3);
+
+    // ---- epilogue -----------------------------------------------------------------------------
+    // accumulator element e of tile (mt, nt): row 8*(e/4) + 4*h + e%4, column r32 of the tile
+    const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
+    // per-column factor (undoes the column normalisation, applies alpha and wcscales) and bias
+    float colf[4], biasf[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+        const int n = wcol0 + nt * 32 + r32;
+        const bool ok = n < p.N;
+        float cf = ok ? p.colnorm[n] * p.alpha : 0.f;
+        if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
+        colf[nt] = cf;
+        biasf[nt] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+    }
+    // operands of the low-rank up projection for the first 32 ranks, requested in one batch so that
+    // their latency is paid once (further ranks are fetched inside the slab loop)
+    const int nsteps = p.R_up / 16;
+    bf16x8_t la_pre[4][2], lb_pre[4][2];
+    auto load_la = [&](int mt, int s) {
+        const float ls = p.lora_scales[s < 8 ? s : 7];
+        const float4_t *ap = (const float4_t *)(p.lora_act + (size_t)(wrow0 + mt * 32 + r32) * p.R_up + 16 * s + 8 * h);
+        const float4_t v0 = ap[0], v1 = ap[1];
+        u32x4_t w;
+        w[0] = f32_to_bf16_bits(v0[0] * ls) | (f32_to_bf16_bits(v0[1] * ls) << 16);
+        w[1] = f32_to_bf16_bits(v0[2] * ls) | (f32_to_bf16_bits(v0[3] * ls) << 16);
+        w[2] = f32_to_bf16_bits(v1[0] * ls) | (f32_to_bf16_bits(v1[1] * ls) << 16);
+        w[3] = f32_to_bf16_bits(v1[2] * ls) | (f32_to_bf16_bits(v1[3] * ls) << 16);
+        return __builtin_bit_cast(bf16x8_t, w);
+    };
+    auto load_lb = [&](int nt, int s) {
+        const int n = wcol0 + nt * 32 + r32;
+        const u32x4_t bw = n < p.N ? *(const u32x4_t *)(p.lora_up + (size_t)n * p.R_up + 16 * s + 8 * h) : u32x4_t{0, 0, 0, 0};
+        return __builtin_bit_cast(bf16x8_t, bw);
+    };
+    if (nsteps > 0) {
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int s = k < nsteps ? k : 0;
+                la_pre[t][k] = load_la(t, s);
+                lb_pre[t][k] = load_lb(t, s);
+            }
+    }
+
+    // reciprocal smoothing factors of the next layer for the 32 columns this lane quantizes
+    // (work item of the quantizing pass: row = item / 4, 32-column quarter = item % 4 = lane % 4)
+    float nrs[32];
+    if (NEXT && p.qout) {
+        const float4_t *sp = (const float4_t *)(p.next_smooth_rcp + (wcol0 < p.N ? wcol0 : 0) + (lane & 3) * 32);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float4_t v = sp[i];
+            nrs[4 * i] = v[0]; nrs[4 * i + 1] = v[1]; nrs[4 * i + 2] = v[2]; nrs[4 * i + 3] = v[3];
+        }
+    }
+    uint16_t *slab = (uint16_t *)(lds + wave * (32 * OUT_LD * 2));
+    const int ngroups_out = p.N / 64;
+    // one 32-row slab of the wave tile; instantiated four times with a compile-time slab index (a
+    // pragma-unrolled loop of this size is refused by the unroller, which would push the
+    // accumulators into scratch memory)
+    auto slab_epilogue = [&](auto MT) {
+        constexpr int mt = decltype(MT)::value;
+        // undo the power-of-two normalisation; per-channel scale and bias (EpilogueBias, gemm_base.cuh:710-781)
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const float rn = rownorm[wm * 128 + mt * 32 + 8 * (e / 4) + 4 * h + (e % 4)];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) acc[mt][nt][e] = acc[mt][nt][e] * rn * colf[nt] + biasf[nt];
+        }
+        // low-rank up projection: acc += bf16(lora_act * scale) @ up^T   (lora.cuh:110-241)
+        if (nsteps > 0) {
+#pragma unroll
+            for (int k = 0; k < 2; k++)
+                if (k < nsteps) {
+#pragma unroll
+                    for (int nt = 0; nt < 4; nt++)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(la_pre[mt][k], lb_pre[nt][k], acc[mt][nt], 0, 0, 0);
+                }
+            for (int s2 = 2; s2 < nsteps; s2++) {
+                const bf16x8_t la = load_la(mt, s2);
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(la, load_lb(nt, s2), acc[mt][nt], 0, 0, 0);
+            }
+        }
+        if (NEXT && p.gelu) {
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[mt][nt][e] = gelu_tanh(acc[mt][nt][e]);
+        }
+        // bf16 tile -> per-wave LDS slab (32 rows x 128 columns): every later consumer reads whole rows
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                slab[(8 * (e / 4) + 4 * h + (e % 4)) * OUT_LD + nt * 32 + r32] = (uint16_t)f32_to_bf16_bits(acc[mt][nt][e]);
+        // the slab is private to this wave: LDS operations of one wave complete in order, so only the
+        // compiler has to be kept from reordering across this point (a fence would also wait for the
+        // global stores in flight)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        if (p.out) {  // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores
+#pragma unroll
+            for (int pass = 0; pass < 8; pass++) {
+                const int rr = pass * 4 + (lane >> 4), cc = (lane & 15) * 8;
+                const int m = wrow0 + mt * 32 + rr, n = wcol0 + cc;
+                if (m < p.M_out && n < p.N_out) *(u32x4_t *)(p.out + (size_t)m * p.N_out + n) = *(const u32x4_t *)(slab + rr * OUT_LD + cc);
+            }
+        }
+        if (NEXT && p.next_down && wcol0 < p.N) {
+            // low-rank down projection of the next layer on the bf16 tile (EpilogueLoraDown,
+            // lora.cuh:243-353): this wave's 128 columns are one 128-chunk of the next layer's K
+            const int RT = p.R_down / 16;
+            const int r16 = lane & 15, q = lane >> 4;
+            for (int rt = 0; rt < RT; rt++) {
+                float4_t d[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const bf16x8_t b = p.next_down[((size_t)((wcol0 / 128) * 4 + i) * RT + rt) * 64 + lane];
+#pragma unroll
+                    for (int m2 = 0; m2 < 2; m2++) {
+                        const bf16x8_t a = *(const bf16x8_t *)(slab + (16 * m2 + r16) * OUT_LD + 32 * q + 8 * i);
+                        d[m2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, d[m2], 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int m2 = 0; m2 < 2; m2++)
+#pragma unroll
+                    for (int i2 = 0; i2 < 4; i2++)
+                        atomicAdd(p.next_lora_out + (size_t)(wrow0 + mt * 32 + 16 * m2 + 4 * q + i2) * p.R_down + 16 * rt + r16, d[m2][i2]);
+            }
+        }
+        if (NEXT && p.qout && wcol0 < p.N) {
+            // EpilogueQuantize (gemm_w4a4.cuh:930-1043): shift, smooth, quantize for the next layer
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++) {
+                const int item = pass * 64 + lane;
+                const int rr = item >> 2, qc = item & 3;
+                const u32x4_t *sp = (const u32x4_t *)(slab + rr * OUT_LD + qc * 32);
+                float y[32];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const u32x4_t v = sp[i];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float lo = bits_f32(v[j] << 16), hi = bits_f32(v[j] & 0xFFFF0000u);
+                        if (!FP4) {  // INT4 next layer: unsigned codes after a +0.171875 shift (launch_impl.cuh:286-294)
+                            lo = bf16_bits_to_f32(f32_to_bf16_bits(__fadd_rn(lo, 0.171875f)));
+                            hi = bf16_bits_to_f32(f32_to_bf16_bits(__fadd_rn(hi, 0.171875f)));
+                        }
+                        y[8 * i + 2 * j] = smooth_quotient(lo, nrs[8 * i + 2 * j]);
+                        y[8 * i + 2 * j + 1] = smooth_quotient(hi, nrs[8 * i + 2 * j + 1]);
+                    }
+                }
+                const int m = wrow0 + mt * 32 + rr;
+                const int gidx = (wcol0 + qc * 32) / 64;
+                u32x4_t words;
+                if (!FP4) {
+                    float sc;
+                    quantize_int4_half_group<true>(y, 1, words, sc);
+                    if ((qc & 1) == 0) ((uint16_t *)p.oscales)[(size_t)gidx * p.M_pad + m] = (uint16_t)f32_to_bf16_bits(sc);
+                } else {
+                    uint32_t sc[2];
+                    quantize_nvfp4_two_groups(y, words, sc);
+                    uint16_t *os = (uint16_t *)p.oscales;  // [N/64][M_pad][4]
+                    os[((size_t)gidx * p.M_pad + m) * 2 + (qc & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
+                }
+                *(u32x4_t *)(p.qout + ((size_t)(m / 32) * ngroups_out + gidx) * TILE_BYTES + (m % 32) * 32 + 16 * (qc & 1)) = words;
+            }
+        }
+        // the slab is private to this wave: LDS operations of one wave complete in order, so only the
+        // compiler has to be kept from reordering across this point (a fence would also wait for the
+        // global stores in flight)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_sched_barrier(0);  // keep the four slabs apart: hoisting the next slab's work multiplies live registers
+    };
+    __builtin_amdgcn_sched_barrier(0);
+    slab_epilogue(std::integral_constant<int, 0>{});
+    slab_epilogue(std::integral_constant<int, 1>{});
+    slab_epilogue(std::integral_constant<int, 2>{});
+    slab_epilogue(std::integral_constant<int, 3>{});
+    SVDQ_STAMP(4);
+}
+
+
+template <bool ACT_UNSIGNED, bool FP4, bool NEXT>
+int launch_gemm_variant(const GemmParams &p, int nwg, hipStream_t stream) {
+    auto kern = gemm_w4a4_kernel<ACT_UNSIGNED, FP4, NEXT>;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+    hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), LDS_BYTES, stream, p);
+    return check_launch("gemm_w4a4");
+}
+
+}  // namespace svdq

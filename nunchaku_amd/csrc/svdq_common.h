@@ -58,11 +58,16 @@ __host__ __device__ inline float bits_f32(uint32_t u) {
     v.u = u;
     return v.f;
 }
-// round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs)
+// round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs); on the device this is the hardware
+// conversion (v_cvt_pk_bf16_f32), on the host the usual integer rounding
 __host__ __device__ inline uint32_t f32_to_bf16_bits(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+#else
     uint32_t u = f32_bits(f);
     u += 0x7FFFu + ((u >> 16) & 1u);
     return u >> 16;
+#endif
 }
 
 // Native tile geometry of 4-bit operands (activations and weights alike):
