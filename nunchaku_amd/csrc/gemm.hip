@@ -40,6 +40,8 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     SVDQ_REQUIRE(((uintptr_t)a->act | (uintptr_t)a->wgt | (uintptr_t)a->ascales | (uintptr_t)a->out | (uintptr_t)a->lora_act_in |
                   (uintptr_t)a->lora_up) % 16 == 0, "gemm: pointers must be 16-byte aligned");
     SVDQ_REQUIRE(a->M_pad * a->N < (1ll << 40) && a->K < (1 << 24), "gemm: shape too large");
+    // scale tables are addressed with 32-bit lane offsets
+    SVDQ_REQUIRE((a->K / 64) * a->M_pad * 4 < (1ll << 31) && (a->K / 64) * a->N * 8 < (1ll << 31), "gemm: scale tables too large");
     if (a->fuse_silu) return fail(SVDQ_EUNSUPPORTED, "gemm: fuse_silu is not implemented");
     if (a->fp4 && a->act_unsigned) return fail(SVDQ_EINVAL, "gemm: NVFP4 activations are never unsigned");
     if (a->qout) {
@@ -83,7 +85,12 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     p.next_down = nullptr; p.next_lora_out = nullptr; p.R_down = 0;
 #endif
 
-    const int nwg = (int)(a->M_pad / BM) * (int)((a->N + BN - 1) / BN);
+    // persistent workgroups: one per compute unit, each walking over its share of the output tiles
+    const int ntiles = (int)(a->M_pad / BM) * (int)((a->N + BN - 1) / BN);
+    int dev = 0, ncu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || ncu <= 0)
+        return fail(SVDQ_ELAUNCH, "gemm: cannot query the number of compute units");
+    const int nwg = ntiles < ncu ? ntiles : ncu;
     const bool next = a->qout != nullptr || a->next_lora_down != nullptr;
     if (p.next_lora_out) {  // the low-rank projection for the next layer is accumulated across column blocks
         const int64_t n = a->M_pad * a->R_down;

@@ -38,9 +38,11 @@
 namespace svdq {
 
 #ifdef SVDQ_GEMM_TIMING
-#define SVDQ_STAMP(i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 8 + (i)] = __builtin_readcyclecounter()
+#define SVDQ_STAMP(i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 64 + (i)] = __builtin_readcyclecounter()
+#define SVDQ_STAMP_TILE(t, i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 64 + 8 + (t) * 8 + (i)] = __builtin_readcyclecounter()
 #else
 #define SVDQ_STAMP(i)
+#define SVDQ_STAMP_TILE(t, i)
 #endif
 
 
@@ -102,63 +104,59 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int r32 = lane & 31, h = lane >> 5;
+    const int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    // ---- block coordinates: consecutive ids of one XCD (id % 8) walk down M inside a band of N
+    // ---- persistent workgroup: tiles first, first + stride, ... -------------------------------
+    // Tile ids are remapped so that the 8 XCDs (id % 8) each walk down M inside their own band of N.
     const int mblocks = p.M_pad / BM, nblocks = (p.N + BN - 1) / BN;
-    const int nwg = mblocks * nblocks;
-    int id = blockIdx.x;
-    {
-        const int per_xcd = (nwg + 7) / 8;
-        const int xcd = id % 8, slot = id / 8;
-        const int lin = xcd * per_xcd + slot;
-        // when nwg is not a multiple of 8 some (xcd, slot) pairs fall outside: fall back to identity
-        id = (nwg % 8 == 0) ? lin : id;
-    }
-    const int bm = id % mblocks, bn = id / mblocks;
-    const int m0 = bm * BM, n0 = bn * BN;
+    const int ntiles = mblocks * nblocks;
     const int kgroups = p.K / 64;
-    const int ntiles_total = p.N / 32;
-
-    float *rownorm = (float *)(lds + ROWNORM_OFF);
-    uint32_t *rowmax = (uint32_t *)(lds + ROWMAX_OFF);
-    SVDQ_STAMP(0);
-
-    // ---- prologue: largest activation scale of each of my 256 rows -> power-of-two renormalisation
-    int my_shift;  // thread tid owns row tid of the block when staging scales
-    if (!FP4) {
-        rowmax[tid] = 0;
-        __syncthreads();
-        const int oct = tid & 31, gs = tid >> 5;
-        uint32_t mx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (int g = gs; g < kgroups; g += 8) {
-            const u32x4_t v = *(const u32x4_t *)(p.ascales + (size_t)g * p.M_pad + m0 + 8 * oct);
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                mx[2 * j] = max(mx[2 * j], v[j] & 0x7FFFu);
-                mx[2 * j + 1] = max(mx[2 * j + 1], (v[j] >> 16) & 0x7FFFu);
-            }
+    const int ntiles32 = p.N / 32;
+    const int my_tiles = ((int)blockIdx.x < ntiles) ? (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    auto tile_coords = [&](int seq, int &m0, int &n0) {
+        int id = blockIdx.x + seq * gridDim.x;
+        if (ntiles % 8 == 0) {  // otherwise some (xcd, slot) pairs would fall outside: keep the identity
+            const int per_xcd = ntiles / 8;
+            id = (id % 8) * per_xcd + id / 8;
         }
+        m0 = (id % mblocks) * BM;
+        n0 = (id / mblocks) * BN;
+    };
+
+    int *rowshift = (int *)(lds + SHIFT_OFF);  // [MAX_BATCH][256] power-of-two renormalisation of the rows
+    constexpr uint32_t AS_ELT = FP4 ? 4 : 2, BS_ELT = FP4 ? 8 : 2;  // bytes of scales per (64-group, row / column)
+    const uint32_t as_stride = (uint32_t)p.M_pad * AS_ELT, bs_stride = (uint32_t)p.N * BS_ELT;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+
+    // Everything needed to stage one tile's operands.  All base addresses are wave-uniform (they live
+    // in scalar registers); a lane adds a 32-bit offset.
+    struct TileCtx {
+        int m0, n0, shift;
+        bool col_ok;
+        const uint8_t *a_base[2], *b_base[2], *as_base, *bs_base;
+        uint32_t bs_voff;
+    };
+    auto make_ctx = [&](int seq, int slot) {
+        TileCtx c;
+        tile_coords(seq, c.m0, c.n0);
+        c.shift = rowshift[slot * 256 + tid];  // thread tid stages the scales of row tid
+        c.col_ok = c.n0 + tid < p.N;
 #pragma unroll
-        for (int j = 0; j < 8; j++) atomicMax(&rowmax[8 * oct + j], mx[j]);
-        __syncthreads();
-        const int ex = (int)(rowmax[tid] >> 7);  // biased bf16 exponent of the row maximum
-        my_shift = ex == 0 ? 0 : NORM_TARGET_EXP - (ex - 127);
-    } else {
-        // NVFP4: four e4m3 scales per (row, 64-group) packed in one word; e4m3 patterns of
-        // non-negative values order like unsigned bytes
-        const uint32_t *sp = (const uint32_t *)p.ascales + m0 + tid;
-        uint32_t mx = 0;
-        for (int g = 0; g < kgroups; g++) {
-            const uint32_t v = sp[(size_t)g * p.M_pad];
-            mx = max(max(mx, v & 0x7Fu), max((v >> 8) & 0x7Fu, max((v >> 16) & 0x7Fu, (v >> 24) & 0x7Fu)));
+        for (int j = 0; j < 2; j++) {
+            const int t = ca + 4 * j;
+            const int nt0 = c.n0 / 32;
+            const int tb = nt0 + t < ntiles32 ? nt0 + t : ntiles32 - 1;  // clamped: its scales are zero
+            c.a_base[j] = p.act + (size_t)(c.m0 / 32 + t) * kgroups * TILE_BYTES;
+            c.b_base[j] = p.wgt + (size_t)tb * kgroups * TILE_BYTES;
         }
-        int ex = 0;
-        if (mx) frexpf(e4m3_to_f32(mx), &ex);  // value in [2^(ex-1), 2^ex)
-        my_shift = mx == 0 ? 0 : NORM_TARGET_EXP - (ex - 1);
-    }
-    rownorm[tid] = ldexpf(1.0f, -my_shift);
-    const bool col_ok = n0 + tid < p.N;
-    SVDQ_STAMP(1);
+        // scale sources: INT4 one bf16 / fp16 value per (group, row / column); NVFP4 one word of four
+        // e4m3 (activations) or four fp16 (weights) per (64-group, row / column)
+        c.as_base = (const uint8_t *)p.ascales + (size_t)c.m0 * AS_ELT;
+        c.bs_base = (const uint8_t *)p.wscales + (size_t)c.n0 * BS_ELT;
+        c.bs_voff = (uint32_t)(c.col_ok ? tid : p.N - 1 - c.n0) * BS_ELT;
+        return c;
+    };
+    const uint32_t code_voff = lane * 16, as_voff = tid * AS_ELT;
 
     // ---- staging -----------------------------------------------------------------------------
     // Code tiles go global -> LDS with asynchronous 16-byte copies (no registers, no ds_write);
@@ -168,50 +166,36 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // iteration is exact: group g+4's codes and group g+3's scales are issued at the top of
     // iteration g; the end of iteration g waits for group g+2 (ten newer operations may stay in
     // flight), which iteration g+1 reads.  That leaves three iterations for a copy to land.
-    const int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int mt0 = m0 / 32, nt0 = n0 / 32;
-    const uint8_t *a_src[2], *b_src[2];
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int t = ca + 4 * j;
-        const int tb = nt0 + t < ntiles_total ? nt0 + t : ntiles_total - 1;  // clamped: its scales are zero
-        a_src[j] = p.act + (size_t)(mt0 + t) * kgroups * TILE_BYTES + lane * 16;
-        b_src[j] = p.wgt + (size_t)tb * kgroups * TILE_BYTES + lane * 16;
-    }
-    // scale sources: INT4 one bf16 / fp16 value per (group, row / column); NVFP4 one word of four e4m3
-    // (activations) or four fp16 (weights) per (64-group, row / column)
-    const uint8_t *as_src = (const uint8_t *)p.ascales + (size_t)(m0 + tid) * (FP4 ? 4 : 2);
-    const uint8_t *bs_src = (const uint8_t *)p.wscales + (size_t)(col_ok ? n0 + tid : p.N - 1) * (FP4 ? 8 : 2);
-    const size_t as_stride = (size_t)p.M_pad * (FP4 ? 4 : 2), bs_stride = (size_t)p.N * (FP4 ? 8 : 2);
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-    auto issue_codes = [&](int g) {  // 4 vector-memory operations
+    auto issue_codes = [&](const TileCtx &c, int g) {  // 4 vector-memory operations
         const int gc = g < kgroups ? g : kgroups - 1;  // surplus copies at the tail are never consumed
         const uint32_t dst = lds_base + (g % STAGES) * STAGE_BYTES + ca * TILE_BYTES;
+        const uint32_t voff = (uint32_t)gc * TILE_BYTES + code_voff;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                         :: "s"(dst + STAGE_A + 4 * j * TILE_BYTES), "v"(a_src[j] + (size_t)gc * TILE_BYTES) : "memory");
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                         :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(b_src[j] + (size_t)gc * TILE_BYTES) : "memory");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :: "s"(dst + STAGE_A + 4 * j * TILE_BYTES), "v"(voff), "s"(c.a_base[j]) : "memory");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(voff), "s"(c.b_base[j]) : "memory");
         }
     };
-    auto issue_scales = [&](int g, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
+    auto issue_scales = [&](const TileCtx &c, int g, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
         const int gc = g < kgroups ? g : kgroups - 1;
+        const uint32_t va = (uint32_t)gc * as_stride + as_voff, vb = (uint32_t)gc * bs_stride + c.bs_voff;
         if (!FP4) {
             uint32_t t;
-            asm volatile("global_load_ushort %0, %1, off" : "=v"(ra) : "v"(as_src + gc * as_stride) : "memory");
-            asm volatile("global_load_ushort %0, %1, off" : "=v"(t) : "v"(bs_src + gc * bs_stride) : "memory");
+            asm volatile("global_load_ushort %0, %1, %2" : "=v"(ra) : "v"(va), "s"(c.as_base) : "memory");
+            asm volatile("global_load_ushort %0, %1, %2" : "=v"(t) : "v"(vb), "s"(c.bs_base) : "memory");
             rb[0] = t;
         } else {
-            asm volatile("global_load_dword %0, %1, off" : "=v"(ra) : "v"(as_src + gc * as_stride) : "memory");
-            asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(rb) : "v"(bs_src + gc * bs_stride) : "memory");
+            asm volatile("global_load_dword %0, %1, %2" : "=v"(ra) : "v"(va), "s"(c.as_base) : "memory");
+            asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(rb) : "v"(vb), "s"(c.bs_base) : "memory");
         }
     };
-    auto store_scales = [&](int g, uint32_t ra, u32x2_t rb) {
+    auto store_scales = [&](const TileCtx &c, int g, uint32_t ra, u32x2_t rb) {
         uint8_t *base = lds + (g % STAGES) * STAGE_BYTES;
         if (!FP4) {
-            const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), my_shift);
-            const _Float16 sb = col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb[0]) : (_Float16)0.f;
+            const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), c.shift);
+            const _Float16 sb = c.col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb[0]) : (_Float16)0.f;
             const _Float16 ma = sa * (_Float16)16.f, mb = sb * (_Float16)16.f;
             const _Float16 na = sa * (_Float16)(ACT_UNSIGNED ? -16.f : -24.f), nb = sb * (_Float16)-24.f;
             *(u32x2_t *)(base + STAGE_AS + tid * 16) = u32x2_t{as_u32(half2_t{ma, ma}), as_u32(half2_t{na, na})};
@@ -220,9 +204,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             u32x4_t pa, pb;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const _Float16 sa = (_Float16)ldexpf(e4m3_to_f32((ra >> (8 * j)) & 0x7Fu), my_shift);
+                const _Float16 sa = (_Float16)ldexpf(e4m3_to_f32((ra >> (8 * j)) & 0x7Fu), c.shift);
                 pa[j] = as_u32(half2_t{sa, sa});
-                const uint32_t hb = col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
+                const uint32_t hb = c.col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
                 pb[j] = hb | (hb << 16);
             }
             *(u32x4_t *)(base + STAGE_AS + tid * 16) = pa;
@@ -230,40 +214,42 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         }
     };
 
-    float16_t acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-
-    // prologue: scales of groups 0..2 and codes of groups 0..3
-    uint32_t sa_e, sa_o;  // scale registers in flight: even / odd groups
-    u32x2_t sb_e, sb_o;
-    {
-        uint32_t s0a, s1a;
-        u32x2_t s0b, s1b;
-        issue_scales(0, s0a, s0b);
-        issue_scales(1, s1a, s1b);
-        issue_scales(2, sa_e, sb_e);
-        issue_codes(0);
-        issue_codes(1);
-        issue_codes(2);
-        issue_codes(3);
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(s0a), "+v"(s0b), "+v"(s1a), "+v"(s1b), "+v"(sa_e), "+v"(sb_e) :: "memory");
-        store_scales(0, s0a, s0b);
-        store_scales(1, s1a, s1b);
-    }
-    __syncthreads();
-    SVDQ_STAMP(2);
-
     // conversion constants, pinned in registers (VOP3 cannot take literals; opaque values let the
     // compiler form v_and_or_b32)
     DequantConsts dc;
     dc.magic = 0x3C003C00u;
     dc.mask = 0x03C003C0u;
     asm volatile("" : "+v"(dc.magic), "+s"(dc.mask));
+
+    float16_t acc[4][4];
+    uint32_t sa_e, sa_o;  // scale registers in flight: even / odd groups
+    u32x2_t sb_e, sb_o;
+    uint32_t s0a, s1a;    // scales of groups 0 and 1 of a tile whose first stages are being fetched
+    u32x2_t s0b, s1b;
+    // first stages of a tile: scales of groups 0..2 (group 2 ends up in sa_e / sb_e, where the main loop
+    // expects it) and codes of groups 0..3.  These scale loads are ordinary loads, not asm: they may
+    // stay in flight across a whole epilogue, and only loads the compiler knows about are safe against
+    // register copies and spills made before the data has arrived.
+    auto load_scales_plain = [&](const TileCtx &c, int g, uint32_t &ra, u32x2_t &rb) {
+        const int gc = g < kgroups ? g : kgroups - 1;
+        if (!FP4) {
+            ra = *(const uint16_t *)(c.as_base + (gc * as_stride + as_voff));
+            rb[0] = *(const uint16_t *)(c.bs_base + (gc * bs_stride + c.bs_voff));
+            rb[1] = 0;
+        } else {
+            ra = *(const uint32_t *)(c.as_base + (gc * as_stride + as_voff));
+            rb = *(const u32x2_t *)(c.bs_base + (gc * bs_stride + c.bs_voff));
+        }
+    };
+    auto issue_first_stages = [&](const TileCtx &c) {
+        load_scales_plain(c, 0, s0a, s0b);
+        load_scales_plain(c, 1, s1a, s1b);
+        load_scales_plain(c, 2, sa_e, sb_e);
+        issue_codes(c, 0);
+        issue_codes(c, 1);
+        issue_codes(c, 2);
+        issue_codes(c, 3);
+    };
 
     // Software pipeline over the 16-wide MFMA steps (4 per k-group): while the 16 MFMAs of a step run,
     // the VALU dequantizes the operands of the next step, so a wave never waits on its own
@@ -293,12 +279,12 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     }
 #define SVDQ_MFMA(A, B)                                                                                   \
     _Pragma("unroll") for (int mt = 0; mt < 4; mt++) _Pragma("unroll") for (int nt = 0; nt < 4; nt++)     \
-        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[mt], B[nt], acc[mt][nt], 0, 0, 0);
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[nt], A[mt], acc[mt][nt], 0, 0, 0);
     // one k-group; S_USE holds the scales of group G+2 (issued one iteration ago), S_LOAD receives G+3's
 #define SVDQ_GROUP(G, SA_USE, SB_USE, SA_LOAD, SB_LOAD)                                                   \
     {                                                                                                     \
-        issue_scales((G) + 3, SA_LOAD, SB_LOAD);                                                          \
-        issue_codes((G) + 4);                                                                             \
+        issue_scales(cur, (G) + 3, SA_LOAD, SB_LOAD);                                                     \
+        issue_codes(cur, (G) + 4);                                                                        \
         SVDQ_CONVERT(araw, braw, asc, bsc, 1, a1, b1)                                                     \
         SVDQ_MFMA(a0, b0)                                                                                 \
         SVDQ_CONVERT(araw, braw, asc, bsc, 2, a0, b0)                                                     \
@@ -319,9 +305,77 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
         }                                                                                                 \
         asm volatile("s_waitcnt vmcnt(10)" : "+v"(SA_USE), "+v"(SB_USE) :: "memory");                     \
-        store_scales((G) + 2, SA_USE, SB_USE);                                                            \
+        store_scales(cur, (G) + 2, SA_USE, SB_USE);                                                       \
         __syncthreads();                                                                                  \
     }
+
+  for (int batch0 = 0; batch0 < my_tiles; batch0 += MAX_BATCH) {
+    const int nbatch = my_tiles - batch0 < MAX_BATCH ? my_tiles - batch0 : MAX_BATCH;
+    SVDQ_STAMP(0);
+    // ---- largest activation scale of every row of the batch's tiles -> power-of-two shift that
+    //      moves it into [2^10, 2^11)
+    __syncthreads();  // the previous batch is done with the table
+    if (!FP4) {
+        for (int t = 0; t < nbatch; t++) rowshift[t * 256 + tid] = 0;
+        __syncthreads();
+        const int oct = tid & 31, gs = tid >> 5;
+        for (int t = 0; t < nbatch; t++) {
+            int m0, n0;
+            tile_coords(batch0 + t, m0, n0);
+            uint32_t mx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int g = gs; g < kgroups; g += 8) {
+                const u32x4_t v = *(const u32x4_t *)(p.ascales + (size_t)g * p.M_pad + m0 + 8 * oct);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    mx[2 * j] = max(mx[2 * j], v[j] & 0x7FFFu);
+                    mx[2 * j + 1] = max(mx[2 * j + 1], (v[j] >> 16) & 0x7FFFu);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) atomicMax((uint32_t *)&rowshift[t * 256 + 8 * oct + j], mx[j]);
+        }
+        __syncthreads();
+        for (int t = 0; t < nbatch; t++) {
+            const int ex = rowshift[t * 256 + tid] >> 7;  // biased bf16 exponent of the row maximum
+            rowshift[t * 256 + tid] = ex == 0 ? 0 : NORM_TARGET_EXP - (ex - 127);
+        }
+    } else {
+        // NVFP4: four e4m3 scales per (row, 64-group) packed in one word; e4m3 patterns of
+        // non-negative values order like unsigned bytes
+        for (int t = 0; t < nbatch; t++) {
+            int m0, n0;
+            tile_coords(batch0 + t, m0, n0);
+            const uint32_t *sp = (const uint32_t *)p.ascales + m0 + tid;
+            uint32_t mx = 0;
+            for (int g = 0; g < kgroups; g++) {
+                const uint32_t v = sp[(size_t)g * p.M_pad];
+                mx = max(max(mx, v & 0x7Fu), max((v >> 8) & 0x7Fu, max((v >> 16) & 0x7Fu, (v >> 24) & 0x7Fu)));
+            }
+            int ex = 0;
+            if (mx) frexpf(e4m3_to_f32(mx), &ex);  // value in [2^(ex-1), 2^ex)
+            rowshift[t * 256 + tid] = mx == 0 ? 0 : NORM_TARGET_EXP - (ex - 1);
+        }
+    }
+    __syncthreads();
+    SVDQ_STAMP(1);
+
+    TileCtx cur = make_ctx(batch0, 0);
+    issue_first_stages(cur);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    store_scales(cur, 0, s0a, s0b);
+    store_scales(cur, 1, s1a, s1b);
+    __syncthreads();
+    SVDQ_STAMP(2);
+
+   for (int ti = 0; ti < nbatch; ti++) {
+    const bool have_next = ti + 1 < nbatch;
+    SVDQ_STAMP_TILE(ti, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     read_raw(0, araw, braw, asc, bsc);
     SVDQ_CONVERT(araw, braw, asc, bsc, 0, a0, b0)
@@ -329,9 +383,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         SVDQ_GROUP(g, sa_e, sb_e, sa_o, sb_o)
         SVDQ_GROUP(g + 1, sa_o, sb_o, sa_e, sb_e)
     }
-#undef SVDQ_GROUP
-#undef SVDQ_CONVERT
-#undef SVDQ_MFMA
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // pin the accumulators in the accumulation registers across the loop exit: without this the
     // register allocator may place the 256 copies into ordinary registers inside the loop body
@@ -339,21 +390,30 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                       "+a"(acc[1][2]), "+a"(acc[1][3]), "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]),
                       "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
     __syncthreads();
-    SVDQ_STAMP(3);
+    SVDQ_STAMP_TILE(ti, 1);
+    const int m0 = cur.m0, n0 = cur.n0;
+    const int *tile_shift = rowshift + ti * 256;
+    TileCtx nxt = cur;
+    if (have_next) nxt = make_ctx(batch0 + ti + 1, ti + 1);
 
     // ---- epilogue -----------------------------------------------------------------------------
-    // accumulator element e of tile (mt, nt): row 8*(e/4) + 4*h + e%4, column r32 of the tile
+    // The MFMAs were issued with the weight tile as the first operand, so a lane holds one output ROW
+    // (r32 of the 32-row tile) and accumulator element e is COLUMN 8*(e/4) + 4*h + e%4 of the 32-column
+    // tile: four consecutive elements are four consecutive output columns.
     const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
-    // per-column factor (undoes the column normalisation, applies alpha and wcscales) and bias
-    float colf[4], biasf[4];
+    // per-column factor (undoes the column normalisation, applies alpha and wcscales) and bias of the
+    // wave's 128 columns, tabulated in LDS (EpilogueBias, gemm_base.cuh:710-781)
+    float *coltab = (float *)(lds + TAB_OFF + wave * 1024);  // [128] factors, then [128] biases
+    {
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-        const int n = wcol0 + nt * 32 + r32;
-        const bool ok = n < p.N;
-        float cf = ok ? p.colnorm[n] * p.alpha : 0.f;
-        if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
-        colf[nt] = cf;
-        biasf[nt] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+        for (int j = 0; j < 2; j++) {
+            const int n = wcol0 + 2 * lane + j;
+            const bool ok = n < p.N;
+            float cf = ok ? p.colnorm[n] * p.alpha : 0.f;
+            if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
+            coltab[2 * lane + j] = cf;
+            coltab[128 + 2 * lane + j] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+        }
     }
     // operands of the low-rank up projection for the first 32 ranks, requested in one batch so that
     // their latency is paid once (further ranks are fetched inside the slab loop)
@@ -364,10 +424,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         const float4_t *ap = (const float4_t *)(p.lora_act + (size_t)(wrow0 + mt * 32 + r32) * p.R_up + 16 * s + 8 * h);
         const float4_t v0 = ap[0], v1 = ap[1];
         u32x4_t w;
-        w[0] = f32_to_bf16_bits(v0[0] * ls) | (f32_to_bf16_bits(v0[1] * ls) << 16);
-        w[1] = f32_to_bf16_bits(v0[2] * ls) | (f32_to_bf16_bits(v0[3] * ls) << 16);
-        w[2] = f32_to_bf16_bits(v1[0] * ls) | (f32_to_bf16_bits(v1[1] * ls) << 16);
-        w[3] = f32_to_bf16_bits(v1[2] * ls) | (f32_to_bf16_bits(v1[3] * ls) << 16);
+        w[0] = pack_bf16x2(v0[0] * ls, v0[1] * ls);
+        w[1] = pack_bf16x2(v0[2] * ls, v0[3] * ls);
+        w[2] = pack_bf16x2(v1[0] * ls, v1[1] * ls);
+        w[3] = pack_bf16x2(v1[2] * ls, v1[3] * ls);
         return __builtin_bit_cast(bf16x8_t, w);
     };
     auto load_lb = [&](int nt, int s) {
@@ -385,6 +445,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 lb_pre[t][k] = load_lb(t, s);
             }
     }
+    // everything requested so far has arrived before the next tile's first stages are requested: a
+    // wait on a later request would otherwise also wait for everything issued in between
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    SVDQ_STAMP_TILE(ti, 2);
+    // first stages of the next tile: in flight while this tile's epilogue runs (the LDS stages are
+    // free, the epilogue works in its own slab)
+    if (have_next) issue_first_stages(nxt);
 
     // reciprocal smoothing factors of the next layer for the 32 columns this lane quantizes
     // (work item of the quantizing pass: row = item / 4, 32-column quarter = item % 4 = lane % 4)
@@ -397,48 +465,64 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             nrs[4 * i] = v[0]; nrs[4 * i + 1] = v[1]; nrs[4 * i + 2] = v[2]; nrs[4 * i + 3] = v[3];
         }
     }
-    uint16_t *slab = (uint16_t *)(lds + wave * (32 * OUT_LD * 2));
+    uint16_t *slab = (uint16_t *)(lds + SLAB_OFF + wave * (32 * OUT_LD * 2));
     const int ngroups_out = p.N / 64;
     // one 32-row slab of the wave tile; instantiated four times with a compile-time slab index (a
     // pragma-unrolled loop of this size is refused by the unroller, which would push the
     // accumulators into scratch memory)
     auto slab_epilogue = [&](auto MT) {
         constexpr int mt = decltype(MT)::value;
-        // undo the power-of-two normalisation; per-channel scale and bias (EpilogueBias, gemm_base.cuh:710-781)
+        // the accumulators of this and the later slabs stay in the accumulation registers up to here
+        // (otherwise the register allocator moves all 256 into ordinary registers right after the main
+        // loop and spills everything else)
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-            const float rn = rownorm[wm * 128 + mt * 32 + 8 * (e / 4) + 4 * h + (e % 4)];
+        for (int m2 = mt; m2 < 4; m2++)
+            asm volatile("" : "+a"(acc[m2][0]), "+a"(acc[m2][1]), "+a"(acc[m2][2]), "+a"(acc[m2][3]));
+        // undo the power-of-two normalisation of the lane's row
+        const float rn = ldexpf(1.0f, -tile_shift[wm * 128 + mt * 32 + r32]);
+        float16_t v[4];
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) acc[mt][nt][e] = acc[mt][nt][e] * rn * colf[nt] + biasf[nt];
-        }
-        // low-rank up projection: acc += bf16(lora_act * scale) @ up^T   (lora.cuh:110-241)
+        for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4_t cf = *(const float4_t *)(coltab + nt * 32 + 8 * q + 4 * h);
+                const float4_t bs = *(const float4_t *)(coltab + 128 + nt * 32 + 8 * q + 4 * h);
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf(acc[mt][nt][4 * q + i] * rn, cf[i], bs[i]);
+            }
+        // low-rank up projection: v += up @ bf16(lora_act * scale)^T   (lora.cuh:110-241)
         if (nsteps > 0) {
 #pragma unroll
             for (int k = 0; k < 2; k++)
                 if (k < nsteps) {
 #pragma unroll
                     for (int nt = 0; nt < 4; nt++)
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(la_pre[mt][k], lb_pre[nt][k], acc[mt][nt], 0, 0, 0);
+                        v[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb_pre[nt][k], la_pre[mt][k], v[nt], 0, 0, 0);
                 }
             for (int s2 = 2; s2 < nsteps; s2++) {
                 const bf16x8_t la = load_la(mt, s2);
 #pragma unroll
                 for (int nt = 0; nt < 4; nt++)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(la, load_lb(nt, s2), acc[mt][nt], 0, 0, 0);
+                    v[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_lb(nt, s2), la, v[nt], 0, 0, 0);
             }
         }
         if (NEXT && p.gelu) {
 #pragma unroll
             for (int nt = 0; nt < 4; nt++)
 #pragma unroll
-                for (int e = 0; e < 16; e++) acc[mt][nt][e] = gelu_tanh(acc[mt][nt][e]);
+                for (int e = 0; e < 16; e++) v[nt][e] = gelu_tanh(v[nt][e]);
         }
-        // bf16 tile -> per-wave LDS slab (32 rows x 128 columns): every later consumer reads whole rows
+        // bf16 tile -> per-wave LDS slab (32 rows x 128 columns), four columns per write: every later
+        // consumer reads whole rows
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
 #pragma unroll
-            for (int e = 0; e < 16; e++)
-                slab[(8 * (e / 4) + 4 * h + (e % 4)) * OUT_LD + nt * 32 + r32] = (uint16_t)f32_to_bf16_bits(acc[mt][nt][e]);
+            for (int q = 0; q < 4; q++) {
+                u32x2_t w;
+                w[0] = pack_bf16x2(v[nt][4 * q], v[nt][4 * q + 1]);
+                w[1] = pack_bf16x2(v[nt][4 * q + 2], v[nt][4 * q + 3]);
+                *(u32x2_t *)(slab + r32 * OUT_LD + nt * 32 + 8 * q + 4 * h) = w;
+            }
         // the slab is private to this wave: LDS operations of one wave complete in order, so only the
         // compiler has to be kept from reordering across this point (a fence would also wait for the
         // global stores in flight)
@@ -525,7 +609,26 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     slab_epilogue(std::integral_constant<int, 1>{});
     slab_epilogue(std::integral_constant<int, 2>{});
     slab_epilogue(std::integral_constant<int, 3>{});
-    SVDQ_STAMP(4);
+    SVDQ_STAMP_TILE(ti, 3);
+    if (have_next) {
+        // the code copies of the next tile must have landed.  Only this tile's stores (and, for more
+        // than 32 ranks or the next-layer epilogue, other requests of unknown number) were issued after
+        // them: a bound on that number lets the stores keep draining while the next tile starts
+        if (!NEXT && p.R_up <= 32)
+            asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        cur = nxt;
+        store_scales(cur, 0, s0a, s0b);
+        store_scales(cur, 1, s1a, s1b);
+    }
+    __syncthreads();
+    SVDQ_STAMP_TILE(ti, 4);
+   }  // tiles of the batch
+  }    // batches
+#undef SVDQ_GROUP
+#undef SVDQ_CONVERT
+#undef SVDQ_MFMA
 }
 
 

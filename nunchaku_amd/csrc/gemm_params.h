@@ -15,9 +15,11 @@ constexpr int STAGES = 4;
 constexpr int STAGE_A = 0, STAGE_B = 8192, STAGE_AS = 16384, STAGE_BS = 16384 + 4096;
 constexpr int STAGE_BYTES = 16384 + 8192;
 constexpr int OUT_LD = 136;                // bf16 elements per row of the store-staging slab (128 + pad)
-constexpr int ROWNORM_OFF = STAGES * STAGE_BYTES;  // fp32 [256] row de-normalisation factors
-constexpr int ROWMAX_OFF = ROWNORM_OFF + 1024;     // u32 [256] scratch for the row maximum
-constexpr int LDS_BYTES = ROWMAX_OFF + 1024;
+constexpr int MAX_BATCH = 8;                       // tiles whose row shifts are tabulated at once
+constexpr int SLAB_OFF = STAGES * STAGE_BYTES;     // 4 waves x (32 rows x OUT_LD bf16): epilogue staging
+constexpr int SHIFT_OFF = SLAB_OFF + 4 * 32 * OUT_LD * 2;  // int [MAX_BATCH][256] row renormalisation shifts
+constexpr int TAB_OFF = SHIFT_OFF + MAX_BATCH * 256 * 4;   // 4 waves x float [2][128]: column factors and biases
+constexpr int LDS_BYTES = TAB_OFF + 4 * 1024;
 constexpr int NORM_TARGET_EXP = 10;
 
 

@@ -70,6 +70,12 @@ __host__ __device__ inline uint32_t f32_to_bf16_bits(float f) {
 #endif
 }
 
+// two fp32 -> packed bf16 pair (lo in bits [15:0]), round-to-nearest-even: one v_cvt_pk_bf16_f32
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bf16x2_t));
+}
+
 // Native tile geometry of 4-bit operands (activations and weights alike):
 //   [rows/32][K/64][32 rows][8 words]; word w of a (row, 64-group) holds elements 8w .. 8w+7.
 //   NVFP4: element e of a word in bits [4e, 4e+4) (plain nibbles).
