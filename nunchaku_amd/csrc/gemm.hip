@@ -13,7 +13,64 @@ int launch_gemm_fp4_v4(const GemmParams &p, int nwg, hipStream_t stream);
 int launch_gemm_fp4_v5(const GemmParams &p, int nwg, hipStream_t stream);
 }  // namespace svdq
 
+#include <mutex>
+#include <stdlib.h>
+
 namespace {
+// Workspace for tiles shared between two workgroups, one per (device, stream): launches on one stream
+// run one after the other and can share it, launches on different streams may overlap and must not.
+// It is allocated the first time a launch needs it and kept until the process ends.
+struct Workspace {
+    int dev;
+    hipStream_t stream;
+    uint8_t *ptr;
+    size_t counters_bytes, partials_bytes;
+};
+constexpr int MAX_WORKSPACES = 16;
+Workspace g_ws[MAX_WORKSPACES];
+int g_ws_count = 0;
+std::mutex g_ws_mutex;
+
+__global__ void zero_f32_kernel(float *p, int64_t n);
+
+// returns nullptr (and sets the error text) on failure
+Workspace *get_workspace(int dev, hipStream_t stream, size_t counters_bytes, size_t partials_bytes) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Workspace *w = nullptr;
+    for (int i = 0; i < g_ws_count; i++)
+        if (g_ws[i].dev == dev && g_ws[i].stream == stream) w = &g_ws[i];
+    if (w && w->counters_bytes >= counters_bytes && w->partials_bytes >= partials_bytes) return w;
+    if (!w) {
+        if (g_ws_count == MAX_WORKSPACES) {
+            fail(SVDQ_ELAUNCH, "gemm: more than %d (device, stream) pairs need a shared-tile workspace", MAX_WORKSPACES);
+            return nullptr;
+        }
+        w = &g_ws[g_ws_count];
+        *w = Workspace{dev, stream, nullptr, 0, 0};
+    } else {
+        (void)hipFree(w->ptr);  // waits for the device: no launch is still using it
+        w->ptr = nullptr;
+    }
+    if (counters_bytes < (1u << 18)) counters_bytes = 1u << 18;
+    counters_bytes = (counters_bytes + 255) & ~(size_t)255;
+    uint8_t *ptr = nullptr;
+    hipError_t e = hipMalloc((void **)&ptr, counters_bytes + partials_bytes);
+    if (e != hipSuccess) {
+        fail(SVDQ_ELAUNCH, "gemm: cannot allocate %zu bytes of shared-tile workspace: %s", counters_bytes + partials_bytes, hipGetErrorString(e));
+        w->counters_bytes = w->partials_bytes = 0;
+        return nullptr;
+    }
+    // the arrival counters start at zero (and every launch leaves them at zero); cleared by a kernel on
+    // the caller's stream so that the clearing is ordered before the launch that follows
+    const int64_t n = (int64_t)(counters_bytes / 4);
+    hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, stream, (float *)ptr, n);
+    w->ptr = ptr;
+    w->counters_bytes = counters_bytes;
+    w->partials_bytes = partials_bytes;
+    if (w == &g_ws[g_ws_count]) g_ws_count++;
+    return w;
+}
+
 __global__ void zero_f32_kernel(float *p, int64_t n) {
     const int64_t i = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) * 4;
     if (i + 3 < n) *(float4_t *)(p + i) = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -44,6 +101,9 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     SVDQ_REQUIRE((a->K / 64) * a->M_pad * 4 < (1ll << 31) && (a->K / 64) * a->N * 8 < (1ll << 31), "gemm: scale tables too large");
     if (a->fuse_silu) return fail(SVDQ_EUNSUPPORTED, "gemm: fuse_silu is not implemented");
     if (a->fp4 && a->act_unsigned) return fail(SVDQ_EINVAL, "gemm: NVFP4 activations are never unsigned");
+    // INT4 adds the low-rank projection before scaling, which is exact only for power-of-two column factors
+    // (the reference asserts alpha == 1 for INT4, gemm_w4a4_launch_impl.cuh:107, and only NVFP4 layers carry wcscales)
+    if (!a->fp4 && (a->alpha != 1.0f || a->wcscales)) return fail(SVDQ_EUNSUPPORTED, "gemm: alpha != 1 and wcscales are NVFP4-only");
     if (a->qout) {
         SVDQ_REQUIRE(a->oscales && a->next_smooth_rcp, "gemm: qout needs oscales and next_smooth_rcp");
         SVDQ_REQUIRE(((uintptr_t)a->qout | (uintptr_t)a->next_smooth_rcp) % 16 == 0, "gemm: qout pointers must be 16-byte aligned");
@@ -90,7 +150,20 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     int dev = 0, ncu = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || ncu <= 0)
         return fail(SVDQ_ELAUNCH, "gemm: cannot query the number of compute units");
-    const int nwg = ntiles < ncu ? ntiles : ncu;
+    int nwg = ntiles < ncu ? ntiles : ncu;
+    if (getenv("SVDQ_GEMM_NO_SHARED_TILES")) {  // whole tiles only: the largest workgroup count that divides the tile count
+        while (ntiles % nwg != 0) nwg--;
+    }
+    // the work is split evenly in units of two k-groups; unless the tile count is a multiple of the
+    // workgroup count, some tiles are then shared by two workgroups and need the workspace
+    p.partials = nullptr;
+    p.counters = nullptr;
+    if (ntiles % nwg != 0) {
+        Workspace *w = get_workspace(dev, (hipStream_t)stream, (size_t)ntiles * 4, (size_t)2 * nwg * 256 * 64 * 16);
+        if (!w) return SVDQ_ELAUNCH;
+        p.counters = (int *)w->ptr;
+        p.partials = (float *)(w->ptr + w->counters_bytes);
+    }
     const bool next = a->qout != nullptr || a->next_lora_down != nullptr;
     if (p.next_lora_out) {  // the low-rank projection for the next layer is accumulated across column blocks
         const int64_t n = a->M_pad * a->R_down;

@@ -95,32 +95,71 @@ __device__ inline float gelu_tanh(float x) {
     return x * (0.5f + 0.5f * t);
 }
 
+// Partial sums of a tile shared by two workgroups travel through memory with system-scope accesses
+// (sc0 sc1): they bypass the caches that are not coherent between the XCDs, so no cache write-back or
+// invalidation is needed around them, only completion (vmcnt) before the arrival counter is touched.
+__device__ inline void store_partial(float4_t *dst, float4_t v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(dst), "v"(v) : "memory");
+}
+__device__ inline void load_partial(float4_t &v, const float4_t *src) {  // complete only after a vmcnt wait that names v
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(src) : "memory");
+}
+#define SVDQ_WAIT_LOADS_16(O)                                                                                       \
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(O[0]), "+v"(O[1]), "+v"(O[2]), "+v"(O[3]), "+v"(O[4]), "+v"(O[5]),      \
+                 "+v"(O[6]), "+v"(O[7]), "+v"(O[8]), "+v"(O[9]), "+v"(O[10]), "+v"(O[11]), "+v"(O[12]), "+v"(O[13]), \
+                 "+v"(O[14]), "+v"(O[15]) :: "memory")
+
 // NEXT: the epilogue also prepares the next layer's input (GELU, quantize, low-rank down); the plain
 // variant carries none of that code or of its registers.
 template <bool ACT_UNSIGNED, bool FP4, bool NEXT>
 __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int r32 = lane & 31, h = lane >> 5;
-    const int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // Thread coordinates.  They are re-derived from an opaque copy of the thread index at the top of every
+    // tile (and again for the epilogue): otherwise everything computed from them anywhere in the kernel
+    // is hoisted to the kernel entry and kept in registers, or spilled, across all loops.
+    int tid = threadIdx.x;
+    int lane = tid & 63, wave = tid >> 6;
+    int wm = wave >> 1, wn = wave & 1;
+    int r32 = lane & 31, h = lane >> 5;
+    int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint32_t code_voff = lane * 16, as_voff = tid * (FP4 ? 4 : 2);
+    auto refresh_thread_coordinates = [&]() {
+        int t = threadIdx.x;
+        asm volatile("" : "+v"(t));
+        tid = t; lane = t & 63; wave = t >> 6;
+        wm = wave >> 1; wn = wave & 1; r32 = lane & 31; h = lane >> 5;
+        ca = __builtin_amdgcn_readfirstlane(t >> 6);
+        code_voff = lane * 16; as_voff = t * (FP4 ? 4 : 2);
+    };
 
-    // ---- persistent workgroup: tiles first, first + stride, ... -------------------------------
-    // Tile ids are remapped so that the 8 XCDs (id % 8) each walk down M inside their own band of N.
+    // ---- persistent workgroups, work split in units of two k-groups ----------------------------
+    // The tiles are numbered down M first (consecutive tiles share their weight columns) and every
+    // tile is a run of K/128 units.  Workgroup v (of W) takes the units [U v / W, U (v+1) / W) of the
+    // concatenated run: every workgroup gets the same amount of work whatever the tile count, at the
+    // price that a tile may be shared by two workgroups (never more: the host launches at most as many
+    // workgroups as there are tiles, so a share is at least one tile long).  A shared tile's two
+    // partial sums are combined by whichever workgroup finishes second (see below).
+    // v is blockIdx remapped so that the 8 XCDs (blockIdx % 8) each own one contiguous band of tiles.
     const int mblocks = p.M_pad / BM, nblocks = (p.N + BN - 1) / BN;
     const int ntiles = mblocks * nblocks;
-    const int kgroups = p.K / 64;
+    const int kgroups = p.K / 64, kunits = kgroups / 2;
     const int ntiles32 = p.N / 32;
-    const int my_tiles = ((int)blockIdx.x < ntiles) ? (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
-    auto tile_coords = [&](int seq, int &m0, int &n0) {
-        int id = blockIdx.x + seq * gridDim.x;
-        if (ntiles % 8 == 0) {  // otherwise some (xcd, slot) pairs would fall outside: keep the identity
-            const int per_xcd = ntiles / 8;
-            id = (id % 8) * per_xcd + id / 8;
-        }
-        m0 = (id % mblocks) * BM;
-        n0 = (id / mblocks) * BN;
+    const int nwg = gridDim.x;
+    const int vwg = nwg % 8 == 0 ? ((int)blockIdx.x % 8) * (nwg / 8) + (int)blockIdx.x / 8 : (int)blockIdx.x;
+    const long long units = (long long)ntiles * kunits;
+    const long long u_begin = units * vwg / nwg, u_end = units * (vwg + 1) / nwg;
+    const int first_tile = (int)(u_begin / kunits);
+    const int nseg = u_end > u_begin ? (int)((u_end - 1) / kunits) - first_tile + 1 : 0;
+    // segment s of this workgroup: tile first_tile + s, k-groups [gb, ge)
+    auto segment = [&](int sidx, int &tile, int &gb, int &ge) {
+        tile = first_tile + sidx;
+        const long long t0 = (long long)tile * kunits;
+        gb = sidx == 0 ? 2 * (int)(u_begin - t0) : 0;
+        ge = u_end - t0 < kunits ? 2 * (int)(u_end - t0) : kgroups;
+    };
+    auto tile_coords = [&](int tile, int &m0, int &n0) {
+        m0 = (tile % mblocks) * BM;
+        n0 = (tile / mblocks) * BN;
     };
 
     int *rowshift = (int *)(lds + SHIFT_OFF);  // [MAX_BATCH][256] power-of-two renormalisation of the rows
@@ -131,14 +170,30 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // Everything needed to stage one tile's operands.  All base addresses are wave-uniform (they live
     // in scalar registers); a lane adds a 32-bit offset.
     struct TileCtx {
+        int tile, gb, ge;  // k-groups [gb, ge) of the tile
         int m0, n0, shift;
         bool col_ok;
         const uint8_t *a_base[2], *b_base[2], *as_base, *bs_base;
         uint32_t bs_voff;
     };
-    auto make_ctx = [&](int seq, int slot) {
+    // follow: the segment after the one given by prev_* (the next tile, from its first k-group), without divisions
+    auto make_ctx = [&](int sidx, int slot, int tid, bool follow, int prev_tile, int prev_m0, int prev_n0) {
         TileCtx c;
-        tile_coords(seq, c.m0, c.n0);
+        if (follow) {
+            c.tile = prev_tile + 1;
+            c.gb = 0;
+            const long long left = u_end - (long long)c.tile * kunits;
+            c.ge = left < kunits ? 2 * (int)left : kgroups;
+            c.m0 = prev_m0 + BM;
+            c.n0 = prev_n0;
+            if (c.m0 == p.M_pad) {
+                c.m0 = 0;
+                c.n0 += BN;
+            }
+        } else {
+            segment(sidx, c.tile, c.gb, c.ge);
+            tile_coords(c.tile, c.m0, c.n0);
+        }
         c.shift = rowshift[slot * 256 + tid];  // thread tid stages the scales of row tid
         c.col_ok = c.n0 + tid < p.N;
 #pragma unroll
@@ -156,7 +211,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         c.bs_voff = (uint32_t)(c.col_ok ? tid : p.N - 1 - c.n0) * BS_ELT;
         return c;
     };
-    const uint32_t code_voff = lane * 16, as_voff = tid * AS_ELT;
 
     // ---- staging -----------------------------------------------------------------------------
     // Code tiles go global -> LDS with asynchronous 16-byte copies (no registers, no ds_write);
@@ -166,9 +220,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // iteration is exact: group g+4's codes and group g+3's scales are issued at the top of
     // iteration g; the end of iteration g waits for group g+2 (ten newer operations may stay in
     // flight), which iteration g+1 reads.  That leaves three iterations for a copy to land.
-    auto issue_codes = [&](const TileCtx &c, int g) {  // 4 vector-memory operations
-        const int gc = g < kgroups ? g : kgroups - 1;  // surplus copies at the tail are never consumed
-        const uint32_t dst = lds_base + (g % STAGES) * STAGE_BYTES + ca * TILE_BYTES;
+    // (l counts the k-groups of the segment; the stage is l % STAGES, the source group c.gb + l)
+    auto issue_codes = [&](const TileCtx &c, int l) {  // 4 vector-memory operations
+        const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;  // surplus copies at the tail are never consumed
+        const uint32_t dst = lds_base + (l % STAGES) * STAGE_BYTES + ca * TILE_BYTES;
         const uint32_t voff = (uint32_t)gc * TILE_BYTES + code_voff;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
@@ -178,8 +233,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                          :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(voff), "s"(c.b_base[j]) : "memory");
         }
     };
-    auto issue_scales = [&](const TileCtx &c, int g, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
-        const int gc = g < kgroups ? g : kgroups - 1;
+    auto issue_scales = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
+        const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
         const uint32_t va = (uint32_t)gc * as_stride + as_voff, vb = (uint32_t)gc * bs_stride + c.bs_voff;
         if (!FP4) {
             uint32_t t;
@@ -230,8 +285,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // expects it) and codes of groups 0..3.  These scale loads are ordinary loads, not asm: they may
     // stay in flight across a whole epilogue, and only loads the compiler knows about are safe against
     // register copies and spills made before the data has arrived.
-    auto load_scales_plain = [&](const TileCtx &c, int g, uint32_t &ra, u32x2_t &rb) {
-        const int gc = g < kgroups ? g : kgroups - 1;
+    auto load_scales_plain = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {
+        const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
         if (!FP4) {
             ra = *(const uint16_t *)(c.as_base + (gc * as_stride + as_voff));
             rb[0] = *(const uint16_t *)(c.bs_base + (gc * bs_stride + c.bs_voff));
@@ -309,9 +364,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         __syncthreads();                                                                                  \
     }
 
-  for (int batch0 = 0; batch0 < my_tiles; batch0 += MAX_BATCH) {
-    const int nbatch = my_tiles - batch0 < MAX_BATCH ? my_tiles - batch0 : MAX_BATCH;
+  for (int batch0 = 0; batch0 < nseg; batch0 += MAX_BATCH) {
+    const int nbatch = nseg - batch0 < MAX_BATCH ? nseg - batch0 : MAX_BATCH;
     SVDQ_STAMP(0);
+    {
+    int tid_p = threadIdx.x;  // opaque copy: nothing derived from it is kept in registers beyond this block
+    asm volatile("" : "+v"(tid_p));
+    const int tid = tid_p;
     // ---- largest activation scale of every row of the batch's tiles -> power-of-two shift that
     //      moves it into [2^10, 2^11)
     __syncthreads();  // the previous batch is done with the table
@@ -321,7 +380,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         const int oct = tid & 31, gs = tid >> 5;
         for (int t = 0; t < nbatch; t++) {
             int m0, n0;
-            tile_coords(batch0 + t, m0, n0);
+            tile_coords(first_tile + batch0 + t, m0, n0);
             uint32_t mx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             for (int g = gs; g < kgroups; g += 8) {
                 const u32x4_t v = *(const u32x4_t *)(p.ascales + (size_t)g * p.M_pad + m0 + 8 * oct);
@@ -344,7 +403,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         // non-negative values order like unsigned bytes
         for (int t = 0; t < nbatch; t++) {
             int m0, n0;
-            tile_coords(batch0 + t, m0, n0);
+            tile_coords(first_tile + batch0 + t, m0, n0);
             const uint32_t *sp = (const uint32_t *)p.ascales + m0 + tid;
             uint32_t mx = 0;
             for (int g = 0; g < kgroups; g++) {
@@ -356,10 +415,11 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             rowshift[t * 256 + tid] = mx == 0 ? 0 : NORM_TARGET_EXP - (ex - 1);
         }
     }
+    }
     __syncthreads();
     SVDQ_STAMP(1);
 
-    TileCtx cur = make_ctx(batch0, 0);
+    TileCtx cur = make_ctx(batch0, 0, threadIdx.x, false, 0, 0, 0);
     issue_first_stages(cur);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     store_scales(cur, 0, s0a, s0b);
@@ -370,18 +430,52 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
    for (int ti = 0; ti < nbatch; ti++) {
     const bool have_next = ti + 1 < nbatch;
     SVDQ_STAMP_TILE(ti, 0);
+    refresh_thread_coordinates();
+    // A tile shared with the next workgroup (this one holds its first k-groups, the neighbour the rest):
+    // the neighbour works on it first thing, so its partial sums are normally parked in the workspace by
+    // now.  Then they are the initial value of the accumulators and this workgroup runs the epilogue.
+    // Slots of the workspace: workgroup v parks the tile its share begins in at 2 v, the one it ends in
+    // at 2 v + 1; layout of a slot [64 quads][256 threads] x float4 (a wave's access covers 1 KB).
+    bool preloaded = false;
+    if (cur.gb == 0 && cur.ge != kgroups) {
+        int *flag = (int *)(lds + TAB_OFF);
+        if (tid == 0) *flag = __hip_atomic_load(p.counters + cur.tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        preloaded = *flag != 0;
+        __syncthreads();
+    }
+    if (preloaded) {
+        const float4_t *theirs = (const float4_t *)p.partials + (size_t)(2 * vwg + 2) * (64 * 256) + tid;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 4; i++) {
+            float4_t o[16];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+            for (int k = 0; k < 16; k++) load_partial(o[k], theirs + (i * 16 + k) * 256);
+            SVDQ_WAIT_LOADS_16(o);
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][j][e] = o[j * 4 + e / 4][e % 4];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+    }
 
     read_raw(0, araw, braw, asc, bsc);
     SVDQ_CONVERT(araw, braw, asc, bsc, 0, a0, b0)
-    for (int g = 0; g < kgroups; g += 2) {  // K is a multiple of 128: an even number of groups
-        SVDQ_GROUP(g, sa_e, sb_e, sa_o, sb_o)
-        SVDQ_GROUP(g + 1, sa_o, sb_o, sa_e, sb_e)
+    // the first iteration refills stage 0, which every wave has to have read by then (inside the loop the
+    // barrier that ends an iteration orders the reads of a stage before its refill)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    const int seg_len = cur.ge - cur.gb;  // even: segments begin and end on units of two k-groups
+    for (int l = 0; l < seg_len; l += 2) {
+        SVDQ_GROUP(l, sa_e, sb_e, sa_o, sb_o)
+        SVDQ_GROUP(l + 1, sa_o, sb_o, sa_e, sb_e)
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // pin the accumulators in the accumulation registers across the loop exit: without this the
@@ -391,11 +485,61 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                       "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
     __syncthreads();
     SVDQ_STAMP_TILE(ti, 1);
+    // Thread coordinates for the epilogue, re-derived from an opaque copy of the thread index: nothing
+    // computed from them can be hoisted above the main loop and occupy registers there.
+    int tid_e = threadIdx.x;
+    asm volatile("" : "+v"(tid_e));
+    const int tid = tid_e, lane = tid_e & 63, wave = __builtin_amdgcn_readfirstlane(tid_e >> 6);
+    const int wm = wave >> 1, wn = wave & 1, r32 = lane & 31, h = lane >> 5;
     const int m0 = cur.m0, n0 = cur.n0;
     const int *tile_shift = rowshift + ti * 256;
     TileCtx nxt = cur;
-    if (have_next) nxt = make_ctx(batch0 + ti + 1, ti + 1);
+    if (have_next) nxt = make_ctx(batch0 + ti + 1, ti + 1, tid, true, cur.tile, cur.m0, cur.n0);
 
+    // ---- a tile shared with a neighbour ------------------------------------------------------
+    // Each of the two workgroups holds the sum over its part of K.  Whoever finishes second adds the
+    // other's partial sums (fp32, so the result does not depend on who that is) and runs the epilogue.
+    // Nobody waits: the first to finish parks its accumulators in its slot of the workspace and goes on.
+    bool run_epilogue = true, combine = false;
+    const float4_t *theirs_base = nullptr;
+    if (preloaded) {
+        // the neighbour's sums were the initial value; leave the counter at zero for the next launch
+        if (tid == 0) __hip_atomic_store(p.counters + cur.tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if (cur.gb != 0 || cur.ge != kgroups) {
+        const bool is_head = cur.gb != 0;  // the share begins inside this tile: the neighbour is v - 1
+        float4_t *mine = (float4_t *)p.partials + (size_t)(2 * vwg + (is_head ? 0 : 1)) * (64 * 256) + tid;
+        const float4_t *theirs = (const float4_t *)p.partials + (size_t)(is_head ? 2 * vwg - 1 : 2 * vwg + 2) * (64 * 256) + tid;
+        int *counter = p.counters + cur.tile;
+        int *flag = (int *)(lds + TAB_OFF);  // free here: the column tables are written further down
+        if (tid == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        bool other_done = *flag != 0;
+        __syncthreads();
+        if (!other_done) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        store_partial(mine + ((i * 4 + j) * 4 + q) * 256,
+                                      float4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]});
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the parked sums are in memory before the counter says so
+            __syncthreads();
+            if (tid == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            other_done = *flag != 0;
+            __syncthreads();
+        }
+        run_epilogue = other_done;
+        combine = other_done;
+        if (other_done) {
+            if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+            theirs_base = theirs;
+        }
+    }
+
+    SVDQ_STAMP_TILE(ti, 5);
     // ---- epilogue -----------------------------------------------------------------------------
     // The MFMAs were issued with the weight tile as the first operand, so a lane holds one output ROW
     // (r32 of the 32-row tile) and accumulator element e is COLUMN 8*(e/4) + 4*h + e%4 of the 32-column
@@ -404,7 +548,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // per-column factor (undoes the column normalisation, applies alpha and wcscales) and bias of the
     // wave's 128 columns, tabulated in LDS (EpilogueBias, gemm_base.cuh:710-781)
     float *coltab = (float *)(lds + TAB_OFF + wave * 1024);  // [128] factors, then [128] biases
-    {
+    if (run_epilogue) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int n = wcol0 + 2 * lane + j;
@@ -415,8 +559,15 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             coltab[128 + 2 * lane + j] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
         }
     }
-    // operands of the low-rank up projection for the first 32 ranks, requested in one batch so that
-    // their latency is paid once (further ranks are fetched inside the slab loop)
+    SVDQ_STAMP_TILE(ti, 6);
+    // Low-rank up projection (lora.cuh:110-241): out += bf16(lora_act * scale) @ up^T on the matrix cores.
+    // INT4: the projection is added to the accumulators BEFORE they are scaled.  The accumulators are in
+    // normalised units (out = acc * rn[row] * cf[col] + bias with rn and cf powers of two: alpha is 1 and
+    // there are no per-channel scales), so the operands are divided by rn and cf first; that only changes
+    // their exponents, the bf16 products are the same numbers.  The matrix cores then update the
+    // accumulators in place and the operands are dead before the output pass starts.
+    // NVFP4: cf is not a power of two; the projection is added after the scaling, inside the output pass.
+    constexpr bool LORA_FIRST = !FP4;
     const int nsteps = p.R_up / 16;
     bf16x8_t la_pre[4][2], lb_pre[4][2];
     auto load_la = [&](int mt, int s) {
@@ -435,16 +586,69 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         const u32x4_t bw = n < p.N ? *(const u32x4_t *)(p.lora_up + (size_t)n * p.R_up + 16 * s + 8 * h) : u32x4_t{0, 0, 0, 0};
         return __builtin_bit_cast(bf16x8_t, bw);
     };
-    if (nsteps > 0) {
+    if (run_epilogue && nsteps > 0) {
+        if (LORA_FIRST) {
+            // two 16-rank steps per round; every request of a round is issued before any of its data is
+            // touched, so a round costs one memory latency
+            for (int s0 = 0; s0 < nsteps; s0 += 2) {
+                const bool two = s0 + 1 < nsteps;
+                const int s1 = two ? s0 + 1 : s0;
+                float4_t ra[4][2][2];
+                u32x4_t rb[4][2];
+                float rcf[4], lsr[4];
 #pragma unroll
-        for (int t = 0; t < 4; t++)
+                for (int t = 0; t < 4; t++) {
+                    const float4_t *ap = (const float4_t *)(p.lora_act + (size_t)(wrow0 + t * 32 + r32) * p.R_up + 8 * h);
+                    ra[t][0][0] = ap[4 * s0]; ra[t][0][1] = ap[4 * s0 + 1];
+                    ra[t][1][0] = ap[4 * s1]; ra[t][1][1] = ap[4 * s1 + 1];
+                    const int n = wcol0 + t * 32 + r32;
+                    const bool ok = n < p.N;
+                    const u32x4_t *bp = (const u32x4_t *)(p.lora_up + (size_t)(ok ? n : 0) * p.R_up + 8 * h);
+                    rb[t][0] = bp[2 * s0];
+                    rb[t][1] = bp[2 * s1];
+                    rcf[t] = ok ? __builtin_amdgcn_rcpf(p.colnorm[n]) : 0.f;  // of a power of two: exact
+                    lsr[t] = ldexpf(1.0f, tile_shift[wm * 128 + t * 32 + r32]);
+                }
 #pragma unroll
-            for (int k = 0; k < 2; k++) {
-                const int s = k < nsteps ? k : 0;
-                la_pre[t][k] = load_la(t, s);
-                lb_pre[t][k] = load_lb(t, s);
+                for (int k = 0; k < 2; k++) {
+                    if (k == 1 && !two) break;
+                    const float ls = p.lora_scales[(s0 + k) < 8 ? (s0 + k) : 7];
+                    bf16x8_t la[4], lb[4];
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const float f = ls * lsr[t];
+                        const float4_t v0 = ra[t][k][0], v1 = ra[t][k][1];
+                        u32x4_t w;
+                        w[0] = pack_bf16x2(v0[0] * f, v0[1] * f);
+                        w[1] = pack_bf16x2(v0[2] * f, v0[3] * f);
+                        w[2] = pack_bf16x2(v1[0] * f, v1[1] * f);
+                        w[3] = pack_bf16x2(v1[2] * f, v1[3] * f);
+                        la[t] = __builtin_bit_cast(bf16x8_t, w);
+                        u32x4_t bw = rb[t][k];
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            bw[i] = pack_bf16x2(bits_f32(bw[i] << 16) * rcf[t], bits_f32(bw[i] & 0xFFFF0000u) * rcf[t]);
+                        lb[t] = __builtin_bit_cast(bf16x8_t, bw);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+                        for (int nt = 0; nt < 4; nt++)
+                            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb[nt], la[mt], acc[mt][nt], 0, 0, 0);
+                }
             }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int k = 0; k < 2; k++) {
+                    const int s = k < nsteps ? k : 0;
+                    la_pre[t][k] = load_la(t, s);
+                    lb_pre[t][k] = load_lb(t, s);
+                }
+        }
     }
+    SVDQ_STAMP_TILE(ti, 7);
     // everything requested so far has arrived before the next tile's first stages are requested: a
     // wait on a later request would otherwise also wait for everything issued in between
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -457,7 +661,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // reciprocal smoothing factors of the next layer for the 32 columns this lane quantizes
     // (work item of the quantizing pass: row = item / 4, 32-column quarter = item % 4 = lane % 4)
     float nrs[32];
-    if (NEXT && p.qout) {
+    if (NEXT && p.qout && run_epilogue) {
         const float4_t *sp = (const float4_t *)(p.next_smooth_rcp + (wcol0 < p.N ? wcol0 : 0) + (lane & 3) * 32);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -470,8 +674,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // one 32-row slab of the wave tile; instantiated four times with a compile-time slab index (a
     // pragma-unrolled loop of this size is refused by the unroller, which would push the
     // accumulators into scratch memory)
-    auto slab_epilogue = [&](auto MT) {
+    auto slab_epilogue = [&](auto MT, auto COMBINE_T) {
         constexpr int mt = decltype(MT)::value;
+        constexpr bool COMBINE = decltype(COMBINE_T)::value;  // a tile shared with a neighbour: add its partial sums
         // the accumulators of this and the later slabs stay in the accumulation registers up to here
         // (otherwise the register allocator moves all 256 into ordinary registers right after the main
         // loop and spills everything else)
@@ -480,6 +685,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             asm volatile("" : "+a"(acc[m2][0]), "+a"(acc[m2][1]), "+a"(acc[m2][2]), "+a"(acc[m2][3]));
         // undo the power-of-two normalisation of the lane's row
         const float rn = ldexpf(1.0f, -tile_shift[wm * 128 + mt * 32 + r32]);
+        // (the accumulators are only read from here on: updating them in place makes the register
+        // allocator copy and spill whole tuples)
+        float4_t other[16];
+        if (COMBINE) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) load_partial(other[k], theirs_base + (mt * 16 + k) * 256);
+            SVDQ_WAIT_LOADS_16(other);
+        }
         float16_t v[4];
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
@@ -487,11 +700,16 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             for (int q = 0; q < 4; q++) {
                 const float4_t cf = *(const float4_t *)(coltab + nt * 32 + 8 * q + 4 * h);
                 const float4_t bs = *(const float4_t *)(coltab + 128 + nt * 32 + 8 * q + 4 * h);
+                if (COMBINE) {
+                    const float4_t o = other[nt * 4 + q];
 #pragma unroll
-                for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf(acc[mt][nt][4 * q + i] * rn, cf[i], bs[i]);
+                    for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf((acc[mt][nt][4 * q + i] + o[i]) * rn, cf[i], bs[i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf(acc[mt][nt][4 * q + i] * rn, cf[i], bs[i]);
+                }
             }
-        // low-rank up projection: v += up @ bf16(lora_act * scale)^T   (lora.cuh:110-241)
-        if (nsteps > 0) {
+        if (!LORA_FIRST && nsteps > 0) {
 #pragma unroll
             for (int k = 0; k < 2; k++)
                 if (k < nsteps) {
@@ -605,16 +823,26 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         __builtin_amdgcn_sched_barrier(0);  // keep the four slabs apart: hoisting the next slab's work multiplies live registers
     };
     __builtin_amdgcn_sched_barrier(0);
-    slab_epilogue(std::integral_constant<int, 0>{});
-    slab_epilogue(std::integral_constant<int, 1>{});
-    slab_epilogue(std::integral_constant<int, 2>{});
-    slab_epilogue(std::integral_constant<int, 3>{});
+    if (run_epilogue && !combine) {
+        slab_epilogue(std::integral_constant<int, 0>{}, std::false_type{});
+        slab_epilogue(std::integral_constant<int, 1>{}, std::false_type{});
+        slab_epilogue(std::integral_constant<int, 2>{}, std::false_type{});
+        slab_epilogue(std::integral_constant<int, 3>{}, std::false_type{});
+    } else if (run_epilogue) {
+        slab_epilogue(std::integral_constant<int, 0>{}, std::true_type{});
+        slab_epilogue(std::integral_constant<int, 1>{}, std::true_type{});
+        slab_epilogue(std::integral_constant<int, 2>{}, std::true_type{});
+        slab_epilogue(std::integral_constant<int, 3>{}, std::true_type{});
+    }
     SVDQ_STAMP_TILE(ti, 3);
     if (have_next) {
-        // the code copies of the next tile must have landed.  Only this tile's stores (and, for more
-        // than 32 ranks or the next-layer epilogue, other requests of unknown number) were issued after
-        // them: a bound on that number lets the stores keep draining while the next tile starts
-        if (!NEXT && p.R_up <= 32)
+        // The code copies of the next tile must have landed.  s_waitcnt vmcnt(n) returns once at most n
+        // requests are outstanding, so it proves that the copies are complete only if at least n
+        // requests were issued after them.  That is known for an interior tile of the plain variant:
+        // each wave issues its 32 output stores (none is skipped, no lane is out of range), and leaving
+        // those in flight lets them drain while the next tile starts.  Everywhere else: wait for all.
+        const bool interior = m0 + BM <= p.M_out && n0 + BN <= p.N_out;
+        if (!NEXT && run_epilogue && interior)
             asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
         else
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -41,6 +41,10 @@ struct GemmParams {
     const float *next_smooth_rcp;  // fp32 [N]
     const bf16x8_t *next_down;   // native proj_down of the next layer ([N, R_down])
     float *next_lora_out;        // fp32 [M_pad, R_down], zeroed before the launch, accumulated atomically
+    // tiles shared by two workgroups: parked partial sums (fp32 [2 * workgroups][256 threads][64] x 4)
+    // and one arrival counter per tile (zero between launches)
+    float *partials;
+    int *counters;
     int M_pad, N, K, M_out, N_out, R_up, R_down;
     float alpha;
     float lora_scales[8];
