@@ -751,7 +751,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             for (int pass = 0; pass < 8; pass++) {
                 const int rr = pass * 4 + (lane >> 4), cc = (lane & 15) * 8;
                 const int m = wrow0 + mt * 32 + rr, n = wcol0 + cc;
-                if (m < p.M_out && n < p.N_out) *(u32x4_t *)(p.out + (size_t)m * p.N_out + n) = *(const u32x4_t *)(slab + rr * OUT_LD + cc);
+                if (m < p.M_out && n < p.N_out)  // streaming store: the tile is not read again by this kernel
+                    __builtin_nontemporal_store(*(const u32x4_t *)(slab + rr * OUT_LD + cc), (u32x4_t *)(p.out + (size_t)m * p.N_out + n));
             }
         }
         if (NEXT && p.next_down && wcol0 < p.N) {

@@ -1,9 +1,11 @@
 // Operator 1: activation smoothing + 4-bit quantization + low-rank down projection in one pass
 // over x.  Counterpart of quantize_w4a4_fuse_lora_kernel (src/kernels/zgemm/gemm_w4a4.cuh:1097-1184).
 //
-// Work split: one workgroup (4 waves) owns 16*MT consecutive rows for the whole K extent, so the
+// Work split: one workgroup (NW = 8 waves) owns 16*MT consecutive rows for the whole K extent, so the
 // low-rank projection needs no atomics and no pre-zeroed output.  Wave w walks the 128-column
-// chunks c = w, w+4, ...  Inside a chunk lane (r = lane%16, q = lane/16) holds, for each 16-row
+// chunks c = w, w+NW, ... and requests the activations of its next chunk before it works on the
+// current one: the kernel is bound by memory latency unless enough bytes are in flight per compute
+// unit.  Inside a chunk lane (r = lane%16, q = lane/16) holds, for each 16-row
 // tile, the 32 consecutive columns 128c + 32q + [0, 32) of row r: half of a 64-group (INT4) or two
 // whole 16-groups (NVFP4).  The same registers feed the bf16 MFMA of the low-rank projection
 // (operand slot (q, j) of step i = column 128c + 32q + 8i + j; proj_down is stored in that order).
@@ -34,9 +36,11 @@ struct QuantParams {
     int M, M_pad, K, R;
 };
 
+constexpr int NW = 8;  // waves per workgroup
+
 template <int MT, int RT_MAX, bool FP4>
-__global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) {
-    extern __shared__ float red[];  // [4 waves][MT][RT][64][4]
+__global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams p) {
+    extern __shared__ float red[];  // [NW waves][MT][RT][64][4]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int r = lane & 15, q = lane >> 4;
@@ -50,17 +54,27 @@ __global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) 
 #pragma unroll
         for (int rt = 0; rt < RT_MAX; rt++) acc[mt][rt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int c = wave; c < p.K / 128; c += 4) {
-        const int kbase = 128 * c + 32 * q;
-        // ---- load x: MT tiles x 4 steps x 8 bf16
-        u32x4_t xv[MT][4];
+    // x of one chunk: MT tiles x 4 steps x 8 bf16 per lane
+    auto load_x = [&](int c, u32x4_t (&xv)[MT][4]) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
             const int row = row0 + 16 * mt + r;
-            const u32x4_t *src = (const u32x4_t *)(p.x + (size_t)row * p.K + kbase);
+            const u32x4_t *src = (const u32x4_t *)(p.x + (size_t)row * p.K + 128 * c + 32 * q);
 #pragma unroll
             for (int i = 0; i < 4; i++) xv[mt][i] = row < p.M ? src[i] : u32x4_t{0, 0, 0, 0};
         }
+    };
+    const int nchunks = p.K / 128;
+    u32x4_t xv_next[MT][4];
+    if (wave < nchunks) load_x(wave, xv_next);
+    for (int c = wave; c < nchunks; c += NW) {
+        const int kbase = 128 * c + 32 * q;
+        u32x4_t xv[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) xv[mt][i] = xv_next[mt][i];
+        if (c + NW < nchunks) load_x(c + NW, xv_next);
         // ---- reciprocal smoothing factors of my 32 columns
         float rs[32];
         if (p.smooth_rcp) {
@@ -123,7 +137,7 @@ __global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) 
         }
     }
 
-    // ---- reduce the four waves' partial projections and write lora_act[row][rank]
+    // ---- reduce the waves' partial projections and write lora_act[row][rank]
     if (RT > 0) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
@@ -132,13 +146,13 @@ __global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) 
                 if (rt < RT) *(float4_t *)&red[(((wave * MT + mt) * RT + rt) * 64 + lane) * 4] = acc[mt][rt];
         __syncthreads();
         const int total = 16 * MT * p.R;
-        for (int idx = threadIdx.x; idx < total; idx += 256) {
+        for (int idx = threadIdx.x; idx < total; idx += 64 * NW) {
             const int row = idx / p.R, rank = idx % p.R;
             const int mt = row / 16, rr = row % 16, rt = rank / 16, rc = rank % 16;
             const int src_lane = 16 * (rr / 4) + rc, i = rr % 4;  // 16x16 MFMA result layout
             float sum = 0.f;
 #pragma unroll
-            for (int w = 0; w < 4; w++) sum += red[(((w * MT + mt) * RT + rt) * 64 + src_lane) * 4 + i];
+            for (int w = 0; w < NW; w++) sum += red[(((w * MT + mt) * RT + rt) * 64 + src_lane) * 4 + i];
             p.lora_out[(size_t)(row0 + row) * p.R + rank] = sum;
         }
     }
@@ -146,13 +160,13 @@ __global__ void __launch_bounds__(256) quantize_fuse_lora_kernel(QuantParams p) 
 
 template <int MT, int RT_MAX, bool FP4>
 int launch(const QuantParams &p, hipStream_t stream) {
-    const size_t smem = (size_t)4 * MT * (p.R / 16) * 64 * 4 * sizeof(float);
+    const size_t smem = (size_t)NW * MT * (p.R / 16) * 64 * 4 * sizeof(float);
     auto kern = quantize_fuse_lora_kernel<MT, RT_MAX, FP4>;
     if (smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "quantize: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(kern, dim3(p.M_pad / (16 * MT)), dim3(256), smem, stream, p);
+    hipLaunchKernelGGL(kern, dim3(p.M_pad / (16 * MT)), dim3(64 * NW), smem, stream, p);
     return check_launch("quantize_w4a4_act_fuse_lora");
 }
 
