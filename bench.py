@@ -67,14 +67,24 @@ def main():
     ap.add_argument("--workload", default="flux_mlp_fc1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=512)
-    ap.add_argument("--only", choices=["gemm", "quantize"], default=None,
-                    help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON)")
+    ap.add_argument("--only", choices=["gemm", "quantize", "copy"], default=None,
+                    help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
+                         "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
 
     import torch
+
+    if args.only == "copy":
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(f"copy: {args.steps} device copies of {src.numel()} bytes (reads {src.numel()}, writes {src.numel()})")
+        return
 
     from nunchaku_amd.models.linear import SVDQW4A4Linear
     from oracle import synth

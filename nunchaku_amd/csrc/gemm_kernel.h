@@ -424,6 +424,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     store_scales(cur, 0, s0a, s0b);
     store_scales(cur, 1, s1a, s1b);
+    // the scales of group 2 are used inside the main loop first: name them here, so that the wait the
+    // compiler owes this ordinary load is placed here and never as a full drain inside the loop
+    asm volatile("" : "+v"(sa_e), "+v"(sb_e));
     __syncthreads();
     SVDQ_STAMP(2);
 
@@ -539,7 +542,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         }
     }
 
-    SVDQ_STAMP_TILE(ti, 5);
     // ---- epilogue -----------------------------------------------------------------------------
     // The MFMAs were issued with the weight tile as the first operand, so a lane holds one output ROW
     // (r32 of the 32-row tile) and accumulator element e is COLUMN 8*(e/4) + 4*h + e%4 of the 32-column
@@ -559,7 +561,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             coltab[128 + 2 * lane + j] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
         }
     }
-    SVDQ_STAMP_TILE(ti, 6);
     // Low-rank up projection (lora.cuh:110-241): out += bf16(lora_act * scale) @ up^T on the matrix cores.
     // INT4: the projection is added to the accumulators BEFORE they are scaled.  The accumulators are in
     // normalised units (out = acc * rn[row] * cf[col] + bias with rn and cf powers of two: alpha is 1 and
@@ -648,7 +649,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 }
         }
     }
-    SVDQ_STAMP_TILE(ti, 7);
     // everything requested so far has arrived before the next tile's first stages are requested: a
     // wait on a later request would otherwise also wait for everything issued in between
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -669,6 +669,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             nrs[4 * i] = v[0]; nrs[4 * i + 1] = v[1]; nrs[4 * i + 2] = v[2]; nrs[4 * i + 3] = v[3];
         }
     }
+    const bool interior = m0 + BM <= p.M_out && n0 + BN <= p.N_out;  // the whole tile lies inside the output
     uint16_t *slab = (uint16_t *)(lds + SLAB_OFF + wave * (32 * OUT_LD * 2));
     const int ngroups_out = p.N / 64;
     // one 32-row slab of the wave tile; instantiated four times with a compile-time slab index (a
@@ -693,13 +694,25 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             for (int k = 0; k < 16; k++) load_partial(other[k], theirs_base + (mt * 16 + k) * 256);
             SVDQ_WAIT_LOADS_16(other);
         }
+        // the column factors and biases of a 32-column tile are requested one tile ahead of their use:
+        // fetched right where they are needed, every group of four would pay the full LDS latency
         float16_t v[4];
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++)
+        float4_t cfv[2][4], bsv[2][4];
+        auto load_cols = [&](int nt, float4_t (&cf)[4], float4_t (&bs)[4]) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const float4_t cf = *(const float4_t *)(coltab + nt * 32 + 8 * q + 4 * h);
-                const float4_t bs = *(const float4_t *)(coltab + 128 + nt * 32 + 8 * q + 4 * h);
+                cf[q] = *(const float4_t *)(coltab + nt * 32 + 8 * q + 4 * h);
+                bs[q] = *(const float4_t *)(coltab + 128 + nt * 32 + 8 * q + 4 * h);
+            }
+        };
+        load_cols(0, cfv[0], bsv[0]);
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+            if (nt < 3) load_cols(nt + 1, cfv[(nt + 1) & 1], bsv[(nt + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4_t cf = cfv[nt & 1][q], bs = bsv[nt & 1][q];
                 if (COMBINE) {
                     const float4_t o = other[nt * 4 + q];
 #pragma unroll
@@ -709,6 +722,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                     for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf(acc[mt][nt][4 * q + i] * rn, cf[i], bs[i]);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+        }
         if (!LORA_FIRST && nsteps > 0) {
 #pragma unroll
             for (int k = 0; k < 2; k++)
@@ -746,12 +761,21 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         // global stores in flight)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_wave_barrier();
-        if (p.out) {  // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores
+        // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores.  Streaming stores: the
+        // tile is not read again by this kernel.
+        if (p.out && interior) {  // no bounds to check: all slab reads first, then all stores
+            u32x4_t d[8];
+#pragma unroll
+            for (int pass = 0; pass < 8; pass++) d[pass] = *(const u32x4_t *)(slab + (pass * 4 + (lane >> 4)) * OUT_LD + (lane & 15) * 8);
+            uint16_t *gp = p.out + (size_t)(wrow0 + mt * 32 + (lane >> 4)) * p.N_out + wcol0 + (lane & 15) * 8;
+#pragma unroll
+            for (int pass = 0; pass < 8; pass++) __builtin_nontemporal_store(d[pass], (u32x4_t *)(gp + (size_t)(pass * 4) * p.N_out));
+        } else if (p.out) {
 #pragma unroll
             for (int pass = 0; pass < 8; pass++) {
                 const int rr = pass * 4 + (lane >> 4), cc = (lane & 15) * 8;
                 const int m = wrow0 + mt * 32 + rr, n = wcol0 + cc;
-                if (m < p.M_out && n < p.N_out)  // streaming store: the tile is not read again by this kernel
+                if (m < p.M_out && n < p.N_out)
                     __builtin_nontemporal_store(*(const u32x4_t *)(slab + rr * OUT_LD + cc), (u32x4_t *)(p.out + (size_t)m * p.N_out + n));
             }
         }
@@ -842,7 +866,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         // requests were issued after them.  That is known for an interior tile of the plain variant:
         // each wave issues its 32 output stores (none is skipped, no lane is out of range), and leaving
         // those in flight lets them drain while the next tile starts.  Everywhere else: wait for all.
-        const bool interior = m0 + BM <= p.M_out && n0 + BN <= p.N_out;
         if (!NEXT && run_epilogue && interior)
             asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
         else
@@ -850,6 +873,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         cur = nxt;
         store_scales(cur, 0, s0a, s0b);
         store_scales(cur, 1, s1a, s1b);
+        asm volatile("" : "+v"(sa_e), "+v"(sb_e));  // as above: the compiler's wait for this load belongs here
     }
     __syncthreads();
     SVDQ_STAMP_TILE(ti, 4);
