@@ -31,6 +31,9 @@ WORKLOADS = {
     "c1_small": dict(M=256, K=3072, N=3072, R=32, seed=0),
 }
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, the peak the metric is quoted against
+# HBM-side bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
+# read for a device copy of known size (profiles/hbm_traffic_*.md); only known for the profiled workload
+PROFILED_GEMM_TRAFFIC_BYTES = {"flux_mlp_fc1": (2.0 * 223350 + 1.0 * 224162) * 1024}
 FP16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 
@@ -166,8 +169,8 @@ def main():
             "gemm_main_term_TOPS": 2.0 * M * N * K / (tg_us * 1e-6) / 1e12,
         },
         "roofline": {
-            "kernel": "gemm_w4a4_int4_kernel", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
-            "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": None,
+            "kernel": "gemm_w4a4_kernel<false, false, false>", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
+            "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": PROFILED_GEMM_TRAFFIC_BYTES.get(args.workload),
             "peak_basis": "dense INT8 MFMA (the metric's peak); the kernel issues fp16 MFMA, dense peak 2500",
             "frac_of_fp16_mfma_peak": gemm_tops / FP16_PEAK_TFLOPS,
         },

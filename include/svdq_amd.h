@@ -9,7 +9,8 @@
  * Conventions
  *   - plain pointers to DEVICE memory, sizes as int64_t, no framework types;
  *   - every function only enqueues work on `stream` (a hipStream_t passed as void*) and returns;
- *     no allocation, no synchronisation, no global state: safe to call from several threads;
+ *     no synchronisation; safe to call from several threads.  One exception to "no allocation, no
+ *     global state": svdq_gemm_w4a4 keeps one workspace per (device, stream) pair, see there;
  *   - return value 0 on success, a negative SVDQ_E* code otherwise; arguments are validated before
  *     anything is launched, so a failed call has no side effect;
  *   - `svdq_last_error()` returns a thread-local human-readable message for the last failure.
@@ -105,6 +106,20 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  *   acc * alpha * wcscales + bias -> + low-rank up -> GELU/SiLU -> [low-rank down of the next
  *   layer] -> store bf16 `out` and/or shift + smooth + quantize for the next layer (`qout`).
  * The GELU is applied exactly when `qout` is given (launch_impl.cuh:282-309).
+ *
+ * INT4 calls must have alpha == 1 and no wcscales (the reference asserts alpha == 1 for INT4,
+ * launch_impl.cuh:107, and only NVFP4 layers carry wcscales): SVDQ_EUNSUPPORTED otherwise.
+ *
+ * Workspace: the work is split evenly over one workgroup per compute unit, so an output tile can be
+ * shared by two workgroups, which exchange fp32 partial sums through device memory.  Unless the
+ * number of 256x256 output tiles is a multiple of the number of compute units (or smaller), the
+ * call needs a workspace of 512 KB per compute unit (128 MB on MI355X) plus 4 bytes per tile.  The
+ * library allocates it with hipMalloc the first time a (device, stream) pair needs it (that call is
+ * not capturable into a graph and may synchronise), keeps it until the process ends and reuses it
+ * for every later call on that pair; at most 16 pairs.  Calls on one stream run in order and share
+ * the workspace safely; the same stream must not be used from two threads at once.  Setting the
+ * environment variable SVDQ_GEMM_NO_SHARED_TILES makes every call use whole tiles only (no workspace,
+ * slower when the tile count does not divide evenly).
  * ------------------------------------------------------------------------------------------ */
 typedef struct svdq_gemm_args {
     const void *act;        /* u8 native activation tiles [M_pad, K/2]                              */
