@@ -80,6 +80,13 @@ def test_gemm_rejects_bad_arguments(lib):
     bad = nv.GemmArgs.from_buffer_copy(a)
     bad.fuse_silu = 1
     assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
+    # INT4 takes neither a per-tensor scale nor per-channel scales (NVFP4 only)
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.alpha = 0.5
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.wcscales = 16
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
 
 
 def test_repack_rejects_bad_arguments(lib):
