@@ -375,24 +375,49 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     //      moves it into [2^10, 2^11)
     __syncthreads();  // the previous batch is done with the table
     if (!FP4) {
+        // thread (oct, gs) takes the groups gs, gs + 8, ... of eight rows; the tiles of the batch go side
+        // by side through one loop so that their loads are in flight together (one memory latency per
+        // step, not one per tile and step)
         for (int t = 0; t < nbatch; t++) rowshift[t * 256 + tid] = 0;
         __syncthreads();
         const int oct = tid & 31, gs = tid >> 5;
-        for (int t = 0; t < nbatch; t++) {
-            int m0, n0;
-            tile_coords(first_tile + batch0 + t, m0, n0);
-            uint32_t mx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            for (int g = gs; g < kgroups; g += 8) {
-                const u32x4_t v = *(const u32x4_t *)(p.ascales + (size_t)g * p.M_pad + m0 + 8 * oct);
+        uint32_t mx[MAX_BATCH][8];
+        const uint16_t *src[MAX_BATCH];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    mx[2 * j] = max(mx[2 * j], v[j] & 0x7FFFu);
-                    mx[2 * j + 1] = max(mx[2 * j + 1], (v[j] >> 16) & 0x7FFFu);
-                }
+        for (int t = 0; t < MAX_BATCH; t++) {
+            int m0, n0;
+            tile_coords(first_tile + batch0 + (t < nbatch ? t : 0), m0, n0);
+            src[t] = p.ascales + m0 + 8 * oct;
+#pragma unroll
+            for (int j = 0; j < 8; j++) mx[t][j] = 0;
+        }
+        for (int g = gs; g < kgroups; g += 24) {
+            // three steps of the group loop at once; slots beyond the batch read the batch's first tile
+            // again and steps beyond K the last group: no branches between the loads, all in flight together
+            u32x4_t v[3][MAX_BATCH];
+#pragma unroll
+            for (int u = 0; u < 3; u++) {
+                const int gu = g + 8 * u < kgroups ? g + 8 * u : kgroups - 1;
+#pragma unroll
+                for (int t = 0; t < MAX_BATCH; t++) v[u][t] = *(const u32x4_t *)(src[t] + (size_t)gu * p.M_pad);
             }
 #pragma unroll
-            for (int j = 0; j < 8; j++) atomicMax((uint32_t *)&rowshift[t * 256 + 8 * oct + j], mx[j]);
+            for (int u = 0; u < 3; u++)
+#pragma unroll
+                for (int t = 0; t < MAX_BATCH; t++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        mx[t][2 * j] = max(mx[t][2 * j], v[u][t][j] & 0x7FFFu);
+                        mx[t][2 * j + 1] = max(mx[t][2 * j + 1], (v[u][t][j] >> 16) & 0x7FFFu);
+                    }
+                }
         }
+#pragma unroll
+        for (int t = 0; t < MAX_BATCH; t++)
+            if (t < nbatch) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) atomicMax((uint32_t *)&rowshift[t * 256 + 8 * oct + j], mx[t][j]);
+            }
         __syncthreads();
         for (int t = 0; t < nbatch; t++) {
             const int ex = rowshift[t * 256 + tid] >> 7;  // biased bf16 exponent of the row maximum
@@ -514,10 +539,15 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         const float4_t *theirs = (const float4_t *)p.partials + (size_t)(is_head ? 2 * vwg - 1 : 2 * vwg + 2) * (64 * 256) + tid;
         int *counter = p.counters + cur.tile;
         int *flag = (int *)(lds + TAB_OFF);  // free here: the column tables are written further down
-        if (tid == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        bool other_done = *flag != 0;
-        __syncthreads();
+        // (a look at the counter first saves the parking when the neighbour is already done; not worth a
+        // round trip where that is unlikely: a share begins with its shared tile and ends with the other)
+        bool other_done = false;
+        if (!is_head) {
+            if (tid == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            other_done = *flag != 0;
+            __syncthreads();
+        }
         if (!other_done) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
