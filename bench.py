@@ -38,7 +38,7 @@ FP16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 
 
-def cpu_baseline(layer, x, rows: int, iters: int = 3):
+def cpu_baseline(layer, x, rows: int, iters: int = 20):
     """The oracle's fake-quant layer on the host cores, on the first `rows` rows of the workload."""
     import torch
 
@@ -65,11 +65,11 @@ def cpu_baseline(layer, x, rows: int, iters: int = 3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="flux_mlp_fc1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-rows", type=int, default=512)
+    ap.add_argument("--cpu-rows", type=int, default=4608)
     ap.add_argument("--only", choices=["gemm", "quantize", "copy"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
                          "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters")
