@@ -101,6 +101,13 @@ __device__ inline float gelu_tanh(float x) {
 __device__ inline void store_partial(float4_t *dst, float4_t v) {
     asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(dst), "v"(v) : "memory");
 }
+// The compiler does not know that an asm load completes later: between the load and the s_waitcnt asm that
+// names its destination, the destination must stay untouched.  That holds as long as the register allocator
+// has no reason to copy or spill it there (the regions that use such loads -- the main loop, the hand-over of
+// the neighbour's sums -- are free of spill code; check the ISA when they change: `scratch_` inside them, or
+// a move of a loaded register before its wait, would be the sign).  Compiler-visible loads are not an
+// option in those regions: the compiler answers them with full vmcnt(0) drains inside the main loop, because
+// it cannot see the waits and the copies issued from asm.
 __device__ inline void load_partial(float4_t &v, const float4_t *src) {  // complete only after a vmcnt wait that names v
     asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(src) : "memory");
 }
