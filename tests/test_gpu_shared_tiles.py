@@ -27,11 +27,12 @@ def _inputs(M_pad, K, R, seed):
     return codes, scales, lora_act
 
 
-@pytest.mark.parametrize("M,K,N,R", [(2304, 256, 7680, 32), (4608, 3072, 12288, 32), (2816, 512, 6400, 16)])
+@pytest.mark.parametrize("M,K,N,R", [(2304, 256, 7680, 32), (4608, 3072, 12288, 32), (2816, 512, 6400, 16), (4500, 384, 3840, 32)])
 def test_shared_tiles_match_whole_tiles(dev, M, K, N, R):
     from nunchaku_amd import packing
     from nunchaku_amd.ops import svdq_gemm_w4a4
 
+    M_out, M = M, (M + 255) // 256 * 256  # operands are padded to 256 rows, the output has M_out rows
     ntiles = (M // 256) * ((N + 255) // 256)
     ncu = torch.cuda.get_device_properties(dev).multi_processor_count
     announce(f"shared tiles M={M} K={K} N={N} R={R}: {ntiles} tiles on {ncu} compute units")
@@ -43,7 +44,7 @@ def test_shared_tiles_match_whole_tiles(dev, M, K, N, R):
     dev_ins = [(packing.logical_to_act(c).to(dev), s.to(dev), la.to(dev)) for c, s, la in ins]
 
     def run(i):
-        out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        out = torch.full((M_out, N), float("nan"), dtype=torch.bfloat16, device=dev)
         act, sc, la = dev_ins[i]
         svdq_gemm_w4a4(act=act, wgt=t["qweight"], out=out, ascales=sc, wscales=t["wscales"], lora_act_in=la,
                        lora_up=t["proj_up"], bias=t["bias"])
@@ -68,7 +69,7 @@ def test_shared_tiles_match_whole_tiles(dev, M, K, N, R):
         assert (diff <= tol).all(), f"launch with input {i}: max difference {diff.max().item()} beyond one bf16 ulp"
         assert (diff > 0).float().mean().item() < 1e-3
     # and the oracle, on a row sample
-    rows = torch.randperm(M, generator=torch.Generator().manual_seed(5))[:64]
+    rows = torch.randperm(M_out, generator=torch.Generator().manual_seed(5))[:64]
     c, s, la = ins[1]
     want = olin.gemm_w4a4(quant.dequant_int4(c[rows], s[:, rows]), quant.dequant_int4(layer.wq, layer.ws), bias=layer.bias,
                           lora_act_in=la[rows], lora_up=layer.proj_up)
