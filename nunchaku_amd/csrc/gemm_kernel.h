@@ -715,12 +715,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     auto slab_epilogue = [&](auto MT, auto COMBINE_T) {
         constexpr int mt = decltype(MT)::value;
         constexpr bool COMBINE = decltype(COMBINE_T)::value;  // a tile shared with a neighbour: add its partial sums
-        // the accumulators of this and the later slabs stay in the accumulation registers up to here
-        // (otherwise the register allocator moves all 256 into ordinary registers right after the main
-        // loop and spills everything else)
-#pragma unroll
-        for (int m2 = mt; m2 < 4; m2++)
-            asm volatile("" : "+a"(acc[m2][0]), "+a"(acc[m2][1]), "+a"(acc[m2][2]), "+a"(acc[m2][3]));
         // undo the power-of-two normalisation of the lane's row
         const float rn = ldexpf(1.0f, -tile_shift[wm * 128 + mt * 32 + r32]);
         // (the accumulators are only read from here on: updating them in place makes the register
