@@ -254,14 +254,16 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         }
     };
     auto store_scales = [&](const TileCtx &c, int g, uint32_t ra, u32x2_t rb) {
-        uint8_t *base = lds + (g % STAGES) * STAGE_BYTES;
+        // (row / column tid of the stage tables, addressed through the lane offset that is live anyway:
+        // the main loop has no register to spare for another address)
+        uint8_t *base = lds + (g % STAGES) * STAGE_BYTES + ca * 1024 + code_voff;
         if (!FP4) {
             const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), c.shift);
             const _Float16 sb = c.col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb[0]) : (_Float16)0.f;
             const _Float16 ma = sa * (_Float16)16.f, mb = sb * (_Float16)16.f;
             const _Float16 na = sa * (_Float16)(ACT_UNSIGNED ? -16.f : -24.f), nb = sb * (_Float16)-24.f;
-            *(u32x2_t *)(base + STAGE_AS + tid * 16) = u32x2_t{as_u32(half2_t{ma, ma}), as_u32(half2_t{na, na})};
-            *(u32x2_t *)(base + STAGE_BS + tid * 16) = u32x2_t{as_u32(half2_t{mb, mb}), as_u32(half2_t{nb, nb})};
+            *(u32x2_t *)(base + STAGE_AS) = u32x2_t{as_u32(half2_t{ma, ma}), as_u32(half2_t{na, na})};
+            *(u32x2_t *)(base + STAGE_BS) = u32x2_t{as_u32(half2_t{mb, mb}), as_u32(half2_t{nb, nb})};
         } else {
             u32x4_t pa, pb;
 #pragma unroll
@@ -271,8 +273,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 const uint32_t hb = c.col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
                 pb[j] = hb | (hb << 16);
             }
-            *(u32x4_t *)(base + STAGE_AS + tid * 16) = pa;
-            *(u32x4_t *)(base + STAGE_BS + tid * 16) = pb;
+            *(u32x4_t *)(base + STAGE_AS) = pa;
+            *(u32x4_t *)(base + STAGE_BS) = pb;
         }
     };
 
@@ -507,6 +509,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // barrier that ends an iteration orders the reads of a stage before its refill)
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __syncthreads();
+    // The compiler cannot see the waits issued from asm.  If it believes that one of its own loads (the
+    // next-layer epilogue has many) might still be in flight here, it protects the registers the loop's
+    // asm loads write with a full vmcnt(0) drain at the top of every iteration.  A wait through the
+    // builtin, which its bookkeeping understands, settles that before the loop.  In these variants the
+    // hand-over has waited for everything already; the plain INT4 variant, whose hand-over leaves output
+    // stores in flight on purpose, does not need it.
+    if (NEXT || FP4) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt unconstrained
     const int seg_len = cur.ge - cur.gb;  // even: segments begin and end on units of two k-groups
     for (int l = 0; l < seg_len; l += 2) {
         SVDQ_GROUP(l, sa_e, sb_e, sa_o, sb_o)
