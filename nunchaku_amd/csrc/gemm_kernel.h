@@ -286,6 +286,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     asm volatile("" : "+v"(dc.magic), "+s"(dc.mask));
 
     float16_t acc[4][4];
+    int coltab_n0 = -1;  // first column of the tile whose column tables are in LDS (wave-uniform)
     uint32_t sa_e, sa_o;  // scale registers in flight: even / odd groups
     u32x2_t sb_e, sb_o;
     uint32_t s0a, s1a;    // scales of groups 0 and 1 of a tile whose first stages are being fetched
@@ -475,7 +476,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // at 2 v + 1; layout of a slot [64 quads][256 threads] x float4 (a wave's access covers 1 KB).
     bool preloaded = false;
     if (cur.gb == 0 && cur.ge != kgroups) {
-        int *flag = (int *)(lds + TAB_OFF);
+        int *flag = (int *)(lds + FLAG_OFF);
         if (tid == 0) *flag = __hip_atomic_load(p.counters + cur.tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         preloaded = *flag != 0;
@@ -554,7 +555,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         float4_t *mine = (float4_t *)p.partials + (size_t)(2 * vwg + (is_head ? 0 : 1)) * (64 * 256) + tid;
         const float4_t *theirs = (const float4_t *)p.partials + (size_t)(is_head ? 2 * vwg - 1 : 2 * vwg + 2) * (64 * 256) + tid;
         int *counter = p.counters + cur.tile;
-        int *flag = (int *)(lds + TAB_OFF);  // free here: the column tables are written further down
+        int *flag = (int *)(lds + FLAG_OFF);
         // (a look at the counter first saves the parking when the neighbour is already done; not worth a
         // round trip where that is unlikely: a share begins with its shared tile and ends with the other)
         bool other_done = false;
@@ -595,8 +596,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
     // per-column factor (undoes the column normalisation, applies alpha and wcscales) and bias of the
     // wave's 128 columns, tabulated in LDS (EpilogueBias, gemm_base.cuh:710-781)
+    // (kept across tiles: consecutive tiles of a workgroup mostly lie in the same 256 columns)
     float *coltab = (float *)(lds + TAB_OFF + wave * 1024);  // [128] factors, then [128] biases
-    if (run_epilogue) {
+    if (run_epilogue && n0 != coltab_n0) {
+        coltab_n0 = n0;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int n = wcol0 + 2 * lane + j;

@@ -19,7 +19,8 @@ constexpr int MAX_BATCH = 8;                       // tiles whose row shifts are
 constexpr int SLAB_OFF = STAGES * STAGE_BYTES;     // 4 waves x (32 rows x OUT_LD bf16): epilogue staging
 constexpr int SHIFT_OFF = SLAB_OFF + 4 * 32 * OUT_LD * 2;  // int [MAX_BATCH][256] row renormalisation shifts
 constexpr int TAB_OFF = SHIFT_OFF + MAX_BATCH * 256 * 4;   // 4 waves x float [2][128]: column factors and biases
-constexpr int LDS_BYTES = TAB_OFF + 4 * 1024;
+constexpr int FLAG_OFF = TAB_OFF + 4 * 1024;               // one word: a thread's reading of an arrival counter, for all
+constexpr int LDS_BYTES = FLAG_OFF + 16;
 constexpr int NORM_TARGET_EXP = 10;
 
 
