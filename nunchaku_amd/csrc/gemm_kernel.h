@@ -98,23 +98,20 @@ __device__ inline float gelu_tanh(float x) {
 // Partial sums of a tile shared by two workgroups travel through memory with system-scope accesses
 // (sc0 sc1): they bypass the caches that are not coherent between the XCDs, so no cache write-back or
 // invalidation is needed around them, only completion (vmcnt) before the arrival counter is touched.
-__device__ inline void store_partial(float4_t *dst, float4_t v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(dst), "v"(v) : "memory");
+// Raw buffer intrinsics carry the cache policy and are ordinary compiler-visible memory operations: the
+// compiler places the waits for the loaded registers itself (a register that an asm load is still going to
+// write is not safe from compiler-made copies).  `slot` is the wave-uniform start of a workspace slot (the
+// descriptor lives in scalar registers); layout of a slot [64 quads][256 threads] x float4.
+constexpr int PARTIAL_SC0_SC1 = 0x11;  // aux bits of the buffer intrinsics on gfx940+: sc0 = 1, sc1 = 16
+__device__ inline __amdgpu_buffer_rsrc_t partial_rsrc(const float4_t *slot) {
+    return __builtin_amdgcn_make_buffer_rsrc((void *)slot, 0, 64 * 256 * 16, 0x00020000);
 }
-// The compiler does not know that an asm load completes later: between the load and the s_waitcnt asm that
-// names its destination, the destination must stay untouched.  That holds as long as the register allocator
-// has no reason to copy or spill it there (the regions that use such loads -- the main loop, the hand-over of
-// the neighbour's sums -- are free of spill code; check the ISA when they change: `scratch_` inside them, or
-// a move of a loaded register before its wait, would be the sign).  Compiler-visible loads are not an
-// option in those regions: the compiler answers them with full vmcnt(0) drains inside the main loop, because
-// it cannot see the waits and the copies issued from asm.
-__device__ inline void load_partial(float4_t &v, const float4_t *src) {  // complete only after a vmcnt wait that names v
-    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(src) : "memory");
+__device__ inline void store_partial(__amdgpu_buffer_rsrc_t r, int tid, int quad, float4_t v) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), r, (quad * 256 + tid) * 16, 0, PARTIAL_SC0_SC1);
 }
-#define SVDQ_WAIT_LOADS_16(O)                                                                                       \
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(O[0]), "+v"(O[1]), "+v"(O[2]), "+v"(O[3]), "+v"(O[4]), "+v"(O[5]),      \
-                 "+v"(O[6]), "+v"(O[7]), "+v"(O[8]), "+v"(O[9]), "+v"(O[10]), "+v"(O[11]), "+v"(O[12]), "+v"(O[13]), \
-                 "+v"(O[14]), "+v"(O[15]) :: "memory")
+__device__ inline float4_t load_partial(__amdgpu_buffer_rsrc_t r, int tid, int quad) {
+    return __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r, (quad * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
+}
 
 // NEXT: the epilogue also prepares the next layer's input (GELU, quantize, low-rank down); the plain
 // variant carries none of that code or of its registers.
@@ -222,11 +219,15 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // ---- staging -----------------------------------------------------------------------------
     // Code tiles go global -> LDS with asynchronous 16-byte copies (no registers, no ds_write);
     // the two scale values per thread travel through registers because they are renormalised on the
-    // way.  All vector-memory traffic of the main loop is issued from volatile asm, in a fixed
-    // order and with a fixed count per iteration, so that one hand-placed s_waitcnt vmcnt(N) per
-    // iteration is exact: group g+4's codes and group g+3's scales are issued at the top of
-    // iteration g; the end of iteration g waits for group g+2 (ten newer operations may stay in
-    // flight), which iteration g+1 reads.  That leaves three iterations for a copy to land.
+    // way.  The main loop works on pairs of k-groups with ONE workgroup barrier per pair (a barrier per
+    // group costs 9 % of the loop in waiting for the slowest wave).  At the top of the pair (l, l+1) the
+    // codes and scales of groups l+3 and l+4 are requested; they go into the stages of groups l-1 and l,
+    // which nobody reads any more (group l's operands were taken into registers during group l-1, before
+    // the previous barrier).  The pair itself reads groups l+1 and l+2 from LDS, which were complete at
+    // the previous barrier.  At the end of the pair every wave waits for its own requests (vmcnt(0):
+    // they have had two group times to land), stores the two sets of scales and meets the others at the
+    // barrier.  The loop's vector-memory requests come from volatile asm: the compiler neither reorders
+    // them nor adds waits of its own for them.
     // (l counts the k-groups of the segment; the stage is l % STAGES, the source group c.gb + l)
     auto issue_codes = [&](const TileCtx &c, int l) {  // 4 vector-memory operations
         const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;  // surplus copies at the tail are never consumed
@@ -287,14 +288,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 
     float16_t acc[4][4];
     int coltab_n0 = -1;  // first column of the tile whose column tables are in LDS (wave-uniform)
-    uint32_t sa_e, sa_o;  // scale registers in flight: even / odd groups
+    uint32_t sa_e, sa_o;  // scale registers in flight: first / second group of the pair being requested
     u32x2_t sb_e, sb_o;
-    uint32_t s0a, s1a;    // scales of groups 0 and 1 of a tile whose first stages are being fetched
-    u32x2_t s0b, s1b;
-    // first stages of a tile: scales of groups 0..2 (group 2 ends up in sa_e / sb_e, where the main loop
-    // expects it) and codes of groups 0..3.  These scale loads are ordinary loads, not asm: they may
-    // stay in flight across a whole epilogue, and only loads the compiler knows about are safe against
-    // register copies and spills made before the data has arrived.
+    uint32_t s0a, s1a, s2a;  // scales of groups 0..2 of a tile whose first stages are being fetched
+    u32x2_t s0b, s1b, s2b;
+    // first stages of a tile: scales and codes of groups 0..2.  These scale loads are ordinary loads, not
+    // asm: they may stay in flight across a whole epilogue, and only loads the compiler knows about are
+    // safe against register copies and spills made before the data has arrived.
     auto load_scales_plain = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {
         const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
         if (!FP4) {
@@ -309,11 +309,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     auto issue_first_stages = [&](const TileCtx &c) {
         load_scales_plain(c, 0, s0a, s0b);
         load_scales_plain(c, 1, s1a, s1b);
-        load_scales_plain(c, 2, sa_e, sb_e);
+        load_scales_plain(c, 2, s2a, s2b);
         issue_codes(c, 0);
         issue_codes(c, 1);
         issue_codes(c, 2);
-        issue_codes(c, 3);
     };
 
     // Software pipeline over the 16-wide MFMA steps (4 per k-group): while the 16 MFMAs of a step run,
@@ -345,11 +344,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #define SVDQ_MFMA(A, B)                                                                                   \
     _Pragma("unroll") for (int mt = 0; mt < 4; mt++) _Pragma("unroll") for (int nt = 0; nt < 4; nt++)     \
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[nt], A[mt], acc[mt][nt], 0, 0, 0);
-    // one k-group; S_USE holds the scales of group G+2 (issued one iteration ago), S_LOAD receives G+3's
-#define SVDQ_GROUP(G, SA_USE, SB_USE, SA_LOAD, SB_LOAD)                                                   \
+    // the arithmetic of one k-group: 64 MFMAs and the conversions for the next 64
+#define SVDQ_GROUP(G)                                                                                     \
     {                                                                                                     \
-        issue_scales(cur, (G) + 3, SA_LOAD, SB_LOAD);                                                     \
-        issue_codes(cur, (G) + 4);                                                                        \
         SVDQ_CONVERT(araw, braw, asc, bsc, 1, a1, b1)                                                     \
         SVDQ_MFMA(a0, b0)                                                                                 \
         SVDQ_CONVERT(araw, braw, asc, bsc, 2, a0, b0)                                                     \
@@ -369,9 +366,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
             __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
         }                                                                                                 \
-        asm volatile("s_waitcnt vmcnt(10)" : "+v"(SA_USE), "+v"(SB_USE) :: "memory");                     \
-        store_scales(cur, (G) + 2, SA_USE, SB_USE);                                                       \
-        __syncthreads();                                                                                  \
     }
 
   for (int batch0 = 0; batch0 < nseg; batch0 += MAX_BATCH) {
@@ -459,9 +453,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     store_scales(cur, 0, s0a, s0b);
     store_scales(cur, 1, s1a, s1b);
-    // the scales of group 2 are used inside the main loop first: name them here, so that the wait the
-    // compiler owes this ordinary load is placed here and never as a full drain inside the loop
-    asm volatile("" : "+v"(sa_e), "+v"(sb_e));
+    store_scales(cur, 2, s2a, s2b);
     __syncthreads();
     SVDQ_STAMP(2);
 
@@ -483,18 +475,18 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         __syncthreads();
     }
     if (preloaded) {
-        const float4_t *theirs = (const float4_t *)p.partials + (size_t)(2 * vwg + 2) * (64 * 256) + tid;
+        const __amdgpu_buffer_rsrc_t theirs_rsrc = partial_rsrc((const float4_t *)p.partials + (size_t)(2 * vwg + 2) * (64 * 256));
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             float4_t o[16];
 #pragma unroll
-            for (int k = 0; k < 16; k++) load_partial(o[k], theirs + (i * 16 + k) * 256);
-            SVDQ_WAIT_LOADS_16(o);
+            for (int k = 0; k < 16; k++) o[k] = load_partial(theirs_rsrc, tid, i * 16 + k);
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[i][j][e] = o[j * 4 + e / 4][e % 4];
         }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), stated in a way the compiler's bookkeeping understands
     } else {
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -519,8 +511,16 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     if (NEXT || FP4) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt unconstrained
     const int seg_len = cur.ge - cur.gb;  // even: segments begin and end on units of two k-groups
     for (int l = 0; l < seg_len; l += 2) {
-        SVDQ_GROUP(l, sa_e, sb_e, sa_o, sb_o)
-        SVDQ_GROUP(l + 1, sa_o, sb_o, sa_e, sb_e)
+        issue_scales(cur, l + 3, sa_e, sb_e);
+        issue_scales(cur, l + 4, sa_o, sb_o);
+        issue_codes(cur, l + 3);
+        issue_codes(cur, l + 4);
+        SVDQ_GROUP(l)
+        SVDQ_GROUP(l + 1)
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(sa_e), "+v"(sb_e), "+v"(sa_o), "+v"(sb_o) :: "memory");
+        store_scales(cur, l + 3, sa_e, sb_e);
+        store_scales(cur, l + 4, sa_o, sb_o);
+        __syncthreads();
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // pin the accumulators in the accumulation registers across the loop exit: without this the
@@ -552,8 +552,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         if (tid == 0) __hip_atomic_store(p.counters + cur.tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else if (cur.gb != 0 || cur.ge != kgroups) {
         const bool is_head = cur.gb != 0;  // the share begins inside this tile: the neighbour is v - 1
-        float4_t *mine = (float4_t *)p.partials + (size_t)(2 * vwg + (is_head ? 0 : 1)) * (64 * 256) + tid;
-        const float4_t *theirs = (const float4_t *)p.partials + (size_t)(is_head ? 2 * vwg - 1 : 2 * vwg + 2) * (64 * 256) + tid;
+        float4_t *mine = (float4_t *)p.partials + (size_t)(2 * vwg + (is_head ? 0 : 1)) * (64 * 256);
+        const float4_t *theirs = (const float4_t *)p.partials + (size_t)(is_head ? 2 * vwg - 1 : 2 * vwg + 2) * (64 * 256);
         int *counter = p.counters + cur.tile;
         int *flag = (int *)(lds + FLAG_OFF);
         // (a look at the counter first saves the parking when the neighbour is already done; not worth a
@@ -566,13 +566,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             __syncthreads();
         }
         if (!other_done) {
+            const __amdgpu_buffer_rsrc_t mine_rsrc = partial_rsrc(mine);
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int q = 0; q < 4; q++)
-                        store_partial(mine + ((i * 4 + j) * 4 + q) * 256,
+                        store_partial(mine_rsrc, tid, (i * 4 + j) * 4 + q,
                                       float4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]});
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the parked sums are in memory before the counter says so
             __syncthreads();
@@ -734,8 +735,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         float4_t other[16];
         if (COMBINE) {
 #pragma unroll
-            for (int k = 0; k < 16; k++) load_partial(other[k], theirs_base + (mt * 16 + k) * 256);
-            SVDQ_WAIT_LOADS_16(other);
+            for (int k = 0; k < 16; k++) other[k] = load_partial(partial_rsrc(theirs_base), tid, mt * 16 + k);
         }
         // the column factors and biases of a 32-column tile are requested one tile ahead of their use:
         // fetched right where they are needed, every group of four would pay the full LDS latency
@@ -916,7 +916,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         cur = nxt;
         store_scales(cur, 0, s0a, s0b);
         store_scales(cur, 1, s1a, s1b);
-        asm volatile("" : "+v"(sa_e), "+v"(sb_e));  // as above: the compiler's wait for this load belongs here
+        store_scales(cur, 2, s2a, s2b);
     }
     __syncthreads();
     SVDQ_STAMP_TILE(ti, 4);
