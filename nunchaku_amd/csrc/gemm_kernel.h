@@ -590,6 +590,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         }
     }
 
+    SVDQ_STAMP_TILE(ti, 5);
     // ---- epilogue -----------------------------------------------------------------------------
     // The MFMAs were issued with the weight tile as the first operand, so a lane holds one output ROW
     // (r32 of the 32-row tile) and accumulator element e is COLUMN 8*(e/4) + 4*h + e%4 of the 32-column
@@ -637,6 +638,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         const u32x4_t bw = n < p.N ? *(const u32x4_t *)(p.lora_up + (size_t)n * p.R_up + 16 * s + 8 * h) : u32x4_t{0, 0, 0, 0};
         return __builtin_bit_cast(bf16x8_t, bw);
     };
+    SVDQ_STAMP_TILE(ti, 6);
     if (run_epilogue && nsteps > 0) {
         if (LORA_FIRST) {
             // two 16-rank steps per round; every request of a round is issued before any of its data is
@@ -699,6 +701,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 }
         }
     }
+    SVDQ_STAMP_TILE(ti, 7);
     // everything requested so far has arrived before the next tile's first stages are requested: a
     // wait on a later request would otherwise also wait for everything issued in between
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
