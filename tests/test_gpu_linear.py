@@ -64,31 +64,56 @@ def test_ops_accept_reference_layout_directly(dev):
     check_output(out, make_oracle(layer).forward(x))
 
 
-@pytest.mark.parametrize("name", ["c2_qkv", "c3_fc1"])
-def test_flux_shapes_properties(dev, name):
-    """Full FLUX shapes: bit-exact quantizer against the oracle on a row sample, GEMM checked on a
-    random sample of output rows against the oracle, plus linearity in the bias."""
+def _full_shape_properties(dev, name, sample_rows=192, linearity=True):
+    """One layer at a full-size configuration: the quantizer bit-exact against the oracle on all rows,
+    the GEMM on a random sample of output rows, plus linearity in the bias."""
     from nunchaku_amd import packing
 
     cfg = synth.CONFIGS[name]
     announce(f"linear {name} {cfg}")
-    M, K, N, R = cfg["M"], cfg["K"], cfg["N"], cfg["R"]
-    layer = synth.make_layer(N, K, R, seed=cfg["seed"])
+    M, K, N, R, fp4 = cfg["M"], cfg["K"], cfg["N"], cfg["R"], bool(cfg.get("fp4"))
+    layer = synth.make_layer(N, K, R, seed=cfg["seed"], fp4=fp4)
     x = synth.make_activations(M, K, seed=cfg["seed"])
     m = make_module(layer, dev)
     ref = make_oracle(layer)
+    if fp4:
+        ref.wtscale = float(torch.tensor(layer.wtscale).to(torch.bfloat16))  # the checkpoint stores wtscale as bf16
     qx, asc, la = m.quantize(x.to(dev))
     y = m.forward_quant(qx, asc, la)[:M]
     torch.cuda.synchronize()
     codes, scales, lora = ref.quantize(x)
-    assert torch.equal(packing.act_to_logical(qx.cpu(), K), codes)
-    assert torch.equal(asc.cpu().view(torch.int16), scales.view(torch.int16))
-    assert (la.cpu() - lora).abs().max().item() <= 2e-5 * lora.abs().max().item()
-    rows = torch.randperm(M, generator=torch.Generator().manual_seed(0))[:192]
+    if fp4:
+        assert torch.equal(packing.act_to_logical(qx.cpu(), K, fp4=True).to(torch.uint8), codes)
+        assert torch.equal(packing.scales_to_logical(asc.cpu(), True).view(torch.uint8), scales.view(torch.uint8))
+    else:
+        assert torch.equal(packing.act_to_logical(qx.cpu(), K), codes)
+        assert torch.equal(asc.cpu().view(torch.int16), scales.view(torch.int16))
+    assert (la.cpu()[:M] - lora[:M]).abs().max().item() <= 2e-5 * lora.abs().max().item()
+    assert not torch.isnan(y.float()).any()
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(0))[:sample_rows]
     want = ref.forward_quant(codes[rows], scales[:, rows], lora[rows])
     check_output(y[rows], want)
-    # bias linearity: y(bias) - y(0) == bias up to bf16 rounding of the two outputs
-    m0 = make_module(synth.LogicalLayer(**{**layer.__dict__, "bias": torch.zeros_like(layer.bias)}), dev)
-    y0 = m0.forward_quant(qx, asc, la)[:M]
-    d = (y.float() - y0.float()).cpu() - layer.bias.float()[None, :]
-    assert d.abs().max().item() <= 2 * 2.0**-7 * max(1.0, y.float().abs().max().item())
+    if linearity:
+        # bias linearity: y(bias) - y(0) == bias up to bf16 rounding of the two outputs
+        m0 = make_module(synth.LogicalLayer(**{**layer.__dict__, "bias": torch.zeros_like(layer.bias)}), dev)
+        y0 = m0.forward_quant(qx, asc, la)[:M]
+        d = (y.float() - y0.float()).cpu() - layer.bias.float()[None, :]
+        assert d.abs().max().item() <= 2 * 2.0**-7 * max(1.0, y.float().abs().max().item())
+
+
+@pytest.mark.parametrize("name", ["c2_qkv", "c3_fc1"])
+def test_flux_shapes_properties(dev, name):
+    """Full FLUX shapes (INT4, rank 32)."""
+    _full_shape_properties(dev, name)
+
+
+@pytest.mark.parametrize("name", ["c4_qkv_mlp", "c4_out"])
+def test_nvfp4_flux_shapes_properties(dev, name):
+    """The NVFP4 configurations at full size: M=4608 with (K=3072, N=21504) and (K=15360, N=3072)."""
+    _full_shape_properties(dev, name)
+
+
+def test_batched_rank128_shape_properties(dev):
+    """M=18432 (4 x 4608 tokens), K=3072, N=12288, rank 128: several batches of tiles per workgroup and
+    four rounds of the low-rank up projection."""
+    _full_shape_properties(dev, "c5", sample_rows=128)
