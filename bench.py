@@ -62,6 +62,26 @@ def cpu_baseline(layer, x, rows: int, iters: int = 20):
     }, y
 
 
+def mfma_rate_probe():
+    """Sustained rate of the GEMM's own MFMA instruction in a loop of nothing else (TFLOP/s), with constant
+    and with random operand bits; None if the probe library has not been built."""
+    import ctypes
+
+    from nunchaku_amd import _native as nv
+
+    if not nv.PROBE_LIB_PATH.exists():
+        return None
+    lib = ctypes.CDLL(str(nv.PROBE_LIB_PATH))
+    lib.svdq_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    res = {}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        v = ctypes.c_double(0.0)
+        if lib.svdq_probe_mfma_rate(rnd, 20000, 10, ctypes.byref(v)) != 0:
+            return None
+        res[name] = v.value
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -70,9 +90,10 @@ def main():
     ap.add_argument("--workload", default="flux_mlp_fc1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=4608)
-    ap.add_argument("--only", choices=["gemm", "quantize", "copy"], default=None,
+    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "mfma-rate"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
-                         "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters")
+                         "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters; "
+                         "'mfma-rate' measures the MFMA instruction of the GEMM alone")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -80,6 +101,10 @@ def main():
 
     import torch
 
+    if args.only == "mfma-rate":
+        torch.cuda.init()
+        print(f"mfma-rate: v_mfma_f32_32x32x16_f16 alone, TFLOP/s: {mfma_rate_probe()}")
+        return
     if args.only == "copy":
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(1)
         dst = torch.empty_like(src)
@@ -173,6 +198,9 @@ def main():
             "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": PROFILED_GEMM_TRAFFIC_BYTES.get(args.workload),
             "peak_basis": "dense INT8 MFMA (the metric's peak); the kernel issues fp16 MFMA, dense peak 2500",
             "frac_of_fp16_mfma_peak": gemm_tops / FP16_PEAK_TFLOPS,
+            # what this GPU sustains on the same instruction with no other work (probe_mfma_rate.hip): with
+            # random operand bits the power management lowers the clock, as it does under the GEMM
+            "fp16_mfma_alone_tflops": mfma_rate_probe(),
         },
     }
     if not args.no_cpu:

@@ -18,6 +18,7 @@ import torch
 _PKG_DIR = Path(__file__).resolve().parent
 _CSRC = _PKG_DIR / "csrc"
 LIB_PATH = _PKG_DIR / "libsvdq_amd.so"
+PROBE_LIB_PATH = _PKG_DIR / "libsvdq_probe.so"  # bench.py's MFMA-rate probe (csrc/probe_mfma_rate.hip)
 SOURCES = ["repack.hip", "quantize.hip", "gemm.hip"]
 HIPCC_FLAGS = [
     "-shared", "-fPIC", "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
@@ -91,6 +92,11 @@ def build(verbose: bool = False, extra_flags: tuple[str, ...] = (), lib_path: Pa
                               capture_output=True, text=True)
         if link.returncode != 0:
             raise RuntimeError("hipcc link failed:\n" + link.stderr[-4000:])
+        if lib_path is None:
+            # measurement aid of bench.py, a library of its own: not part of the operator ABI
+            probe = subprocess.run([hipcc, *HIPCC_FLAGS, str(_CSRC / "probe_mfma_rate.hip"), "-o", str(PROBE_LIB_PATH)], capture_output=True, text=True)
+            if probe.returncode != 0:
+                raise RuntimeError("hipcc failed on probe_mfma_rate.hip:\n" + probe.stderr[-4000:])
     if verbose:
         print(f"built {out}")
     return out

@@ -139,3 +139,13 @@ def test_module_mirrors_reference_parameters():
         SVDQW4A4Linear(256, 384, precision="int8")
     lin = torch.nn.Linear(256, 384, dtype=torch.bfloat16)
     assert SVDQW4A4Linear.from_linear(lin, rank=16).rank == 16
+
+
+def test_probe_library_exports_its_entry_point():
+    """bench.py's MFMA-rate probe is a library of its own (not part of the operator ABI); no GPU call here."""
+    import ctypes
+
+    from nunchaku_amd import _native as nv
+
+    assert nv.PROBE_LIB_PATH.exists(), "build with __graft_entry__.build()"
+    assert hasattr(ctypes.CDLL(str(nv.PROBE_LIB_PATH)), "svdq_probe_mfma_rate")
