@@ -153,12 +153,19 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     int nwg = ntiles < ncu ? ntiles : ncu;
     if (getenv("SVDQ_GEMM_NO_SHARED_TILES")) {  // whole tiles only: the largest workgroup count that divides the tile count
         while (ntiles % nwg != 0) nwg--;
+    } else if (ntiles < ncu) {
+        // fewer tiles than compute units: several workgroups per tile, each with at least four units (eight
+        // k-groups) of work, so that the fixed cost of a workgroup and of adding up the parts stays small
+        const long long units = (long long)ntiles * (a->K / 128);
+        long long w = units / 4;
+        if (w > ncu) w = ncu;
+        if (w > nwg) nwg = (int)w;
     }
     // the work is split evenly in units of two k-groups; unless the tile count is a multiple of the
-    // workgroup count, some tiles are then shared by two workgroups and need the workspace
+    // workgroup count, some tiles are then shared by two or more workgroups and need the workspace
     p.partials = nullptr;
     p.counters = nullptr;
-    if (ntiles % nwg != 0) {
+    if (nwg > ntiles || ntiles % nwg != 0) {
         Workspace *w = get_workspace(dev, (hipStream_t)stream, (size_t)ntiles * 4, (size_t)2 * nwg * 256 * 64 * 16);
         if (!w) return SVDQ_ELAUNCH;
         p.counters = (int *)w->ptr;

@@ -126,14 +126,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     int wm = wave >> 1, wn = wave & 1;
     int r32 = lane & 31, h = lane >> 5;
     int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
-    uint32_t code_voff = lane * 16, as_voff = tid * (FP4 ? 4 : 2);
+    uint32_t code_voff = lane * 16, as_voff = lane * (FP4 ? 4 : 2);  // (the wave's part of the scale offset is in as_base)
     auto refresh_thread_coordinates = [&]() {
         int t = threadIdx.x;
         asm volatile("" : "+v"(t));
         tid = t; lane = t & 63; wave = t >> 6;
         wm = wave >> 1; wn = wave & 1; r32 = lane & 31; h = lane >> 5;
         ca = __builtin_amdgcn_readfirstlane(t >> 6);
-        code_voff = lane * 16; as_voff = t * (FP4 ? 4 : 2);
+        code_voff = lane * 16; as_voff = lane * (FP4 ? 4 : 2);
     };
 
     // ---- persistent workgroups, work split in units of two k-groups ----------------------------
@@ -166,6 +166,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         n0 = (tile / mblocks) * BN;
     };
 
+    // the workgroups [lo, hi] whose shares reach into a tile (units [t0, t0 + kunits)); more than two only
+    // when there are fewer tiles than workgroups
+    auto tile_parties = [&](int tile, int &lo, int &hi) {
+        const long long t0 = (long long)tile * kunits, t1 = t0 + kunits;
+        lo = (int)(((t0 + 1) * nwg + units - 1) / units) - 1;  // first v with units (v + 1) / nwg > t0
+        hi = (int)((t1 * nwg - 1) / units);                    // last v with units v / nwg < t1
+    };
     int *rowshift = (int *)(lds + SHIFT_OFF);  // [MAX_BATCH][256] power-of-two renormalisation of the rows
     constexpr uint32_t AS_ELT = FP4 ? 4 : 2, BS_ELT = FP4 ? 8 : 2;  // bytes of scales per (64-group, row / column)
     const uint32_t as_stride = (uint32_t)p.M_pad * AS_ELT, bs_stride = (uint32_t)p.N * BS_ELT;
@@ -210,7 +217,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         }
         // scale sources: INT4 one bf16 / fp16 value per (group, row / column); NVFP4 one word of four
         // e4m3 (activations) or four fp16 (weights) per (64-group, row / column)
-        c.as_base = (const uint8_t *)p.ascales + (size_t)c.m0 * AS_ELT;
+        c.as_base = (const uint8_t *)p.ascales + (size_t)(c.m0 + ca * 64) * AS_ELT;  // row m0 + tid = m0 + 64 ca + lane
         c.bs_base = (const uint8_t *)p.wscales + (size_t)c.n0 * BS_ELT;
         c.bs_voff = (uint32_t)(c.col_ok ? tid : p.N - 1 - c.n0) * BS_ELT;
         return c;
@@ -243,7 +250,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     };
     auto issue_scales = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
         const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
-        const uint32_t va = (uint32_t)gc * as_stride + as_voff, vb = (uint32_t)gc * bs_stride + c.bs_voff;
+        // (the lane's scale offset is derived from the live code offset on the spot: one shift, and no
+        // register of its own across the loop)
+        uint32_t lane_off;
+        if (!FP4)
+            asm volatile("v_lshrrev_b32 %0, 3, %1" : "=v"(lane_off) : "v"(code_voff));
+        else
+            asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(lane_off) : "v"(code_voff));
+        const uint32_t va = (uint32_t)gc * as_stride + lane_off, vb = (uint32_t)gc * bs_stride + c.bs_voff;
         if (!FP4) {
             uint32_t t;
             asm volatile("global_load_ushort %0, %1, %2" : "=v"(ra) : "v"(va), "s"(c.as_base) : "memory");
@@ -467,7 +481,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // Slots of the workspace: workgroup v parks the tile its share begins in at 2 v, the one it ends in
     // at 2 v + 1; layout of a slot [64 quads][256 threads] x float4 (a wave's access covers 1 KB).
     bool preloaded = false;
+    bool two_parties = false;
     if (cur.gb == 0 && cur.ge != kgroups) {
+        int lo, hi;
+        tile_parties(cur.tile, lo, hi);
+        two_parties = hi - lo == 1;
+    }
+    if (two_parties) {
         int *flag = (int *)(lds + FLAG_OFF);
         if (tid == 0) *flag = __hip_atomic_load(p.counters + cur.tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
@@ -536,36 +556,38 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     asm volatile("" : "+v"(tid_e));
     const int tid = tid_e, lane = tid_e & 63, wave = __builtin_amdgcn_readfirstlane(tid_e >> 6);
     const int wm = wave >> 1, wn = wave & 1, r32 = lane & 31, h = lane >> 5;
-    const int m0 = cur.m0, n0 = cur.n0;
+    const int m0 = cur.m0, n0 = cur.n0, tile_e = cur.tile;
     const int *tile_shift = rowshift + ti * 256;
     TileCtx nxt = cur;
     if (have_next) nxt = make_ctx(batch0 + ti + 1, ti + 1, tid, true, cur.tile, cur.m0, cur.n0);
 
-    // ---- a tile shared with a neighbour ------------------------------------------------------
-    // Each of the two workgroups holds the sum over its part of K.  Whoever finishes second adds the
-    // other's partial sums (fp32, so the result does not depend on who that is) and runs the epilogue.
-    // Nobody waits: the first to finish parks its accumulators in its slot of the workspace and goes on.
+    // ---- a tile shared with other workgroups ---------------------------------------------------
+    // Every party holds the sum over its part of K.  Whoever finishes last adds the others' partial sums
+    // (fp32; with two parties the result does not depend on who that is, with more the order of the
+    // additions is fixed: ascending workgroup, own sums last) and runs the epilogue.  Nobody waits: the
+    // others park their accumulators in their slot of the workspace and go on.
     bool run_epilogue = true, combine = false;
-    const float4_t *theirs_base = nullptr;
+    int party_lo = 0, party_hi = -1;  // (worked out here, not ahead of the main loop, where they would occupy registers)
+    if (!preloaded && (cur.gb != 0 || cur.ge != kgroups)) tile_parties(tile_e, party_lo, party_hi);
     if (preloaded) {
         // the neighbour's sums were the initial value; leave the counter at zero for the next launch
         if (tid == 0) __hip_atomic_store(p.counters + cur.tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else if (cur.gb != 0 || cur.ge != kgroups) {
-        const bool is_head = cur.gb != 0;  // the share begins inside this tile: the neighbour is v - 1
+        const bool is_head = cur.gb != 0;  // the share begins inside this tile
+        const int others = party_hi - party_lo;
         float4_t *mine = (float4_t *)p.partials + (size_t)(2 * vwg + (is_head ? 0 : 1)) * (64 * 256);
-        const float4_t *theirs = (const float4_t *)p.partials + (size_t)(is_head ? 2 * vwg - 1 : 2 * vwg + 2) * (64 * 256);
         int *counter = p.counters + cur.tile;
         int *flag = (int *)(lds + FLAG_OFF);
-        // (a look at the counter first saves the parking when the neighbour is already done; not worth a
+        // (a look at the counter first saves the parking when everybody else is already done; not worth a
         // round trip where that is unlikely: a share begins with its shared tile and ends with the other)
-        bool other_done = false;
+        bool last = false;
         if (!is_head) {
             if (tid == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
-            other_done = *flag != 0;
+            last = *flag == others;
             __syncthreads();
         }
-        if (!other_done) {
+        if (!last) {
             const __amdgpu_buffer_rsrc_t mine_rsrc = partial_rsrc(mine);
 #pragma unroll
             for (int i = 0; i < 4; i++)
@@ -579,15 +601,12 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             __syncthreads();
             if (tid == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
-            other_done = *flag != 0;
+            last = *flag == others;
             __syncthreads();
         }
-        run_epilogue = other_done;
-        combine = other_done;
-        if (other_done) {
-            if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-            theirs_base = theirs;
-        }
+        run_epilogue = last;
+        combine = last;
+        if (last && tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
     }
 
     SVDQ_STAMP_TILE(ti, 5);
@@ -738,7 +757,15 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         float4_t other[16];
         if (COMBINE) {
 #pragma unroll
-            for (int k = 0; k < 16; k++) other[k] = load_partial(partial_rsrc(theirs_base), tid, mt * 16 + k);
+            for (int k = 0; k < 16; k++) other[k] = float4_t{0.f, 0.f, 0.f, 0.f};
+            for (int v = party_lo; v <= party_hi; v++) {
+                if (v == vwg) continue;
+                // a workgroup parks the tile its share begins inside at slot 2 v, otherwise at 2 v + 1
+                const bool begins_inside = units * v / nwg > (long long)tile_e * kunits;
+                const __amdgpu_buffer_rsrc_t r = partial_rsrc((const float4_t *)p.partials + (size_t)(2 * v + (begins_inside ? 0 : 1)) * (64 * 256));
+#pragma unroll
+                for (int k = 0; k < 16; k++) other[k] += load_partial(r, tid, mt * 16 + k);
+            }
         }
         // the column factors and biases of a 32-column tile are requested one tile ahead of their use:
         // fetched right where they are needed, every group of four would pay the full LDS latency
