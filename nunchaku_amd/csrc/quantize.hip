@@ -1,11 +1,13 @@
 // Operator 1: activation smoothing + 4-bit quantization + low-rank down projection in one pass
 // over x.  Counterpart of quantize_w4a4_fuse_lora_kernel (src/kernels/zgemm/gemm_w4a4.cuh:1097-1184).
 //
-// Work split: one workgroup (NW = 8 waves) owns 16*MT consecutive rows for the whole K extent, so the
+// Work split: one workgroup (NW waves) owns 16*MT consecutive rows for the whole K extent, so the
 // low-rank projection needs no atomics and no pre-zeroed output.  Wave w walks the 128-column
-// chunks c = w, w+NW, ... and requests the activations of its next chunk before it works on the
-// current one: the kernel is bound by memory latency unless enough bytes are in flight per compute
-// unit.  Inside a chunk lane (r = lane%16, q = lane/16) holds, for each 16-row
+// chunks c = w, w+NW, ... and keeps the activations of its next DEPTH chunks requested while it works
+// on the current one: the kernel is bound by memory latency unless enough bytes are in flight per
+// compute unit.  The reciprocal smoothing factors are copied to LDS once per workgroup, and the
+// low-rank operands of a chunk are requested before its quantization and used after it.  Inside a
+// chunk lane (r = lane%16, q = lane/16) holds, for each 16-row
 // tile, the 32 consecutive columns 128c + 32q + [0, 32) of row r: half of a 64-group (INT4) or two
 // whole 16-groups (NVFP4).  The same registers feed the bf16 MFMA of the low-rank projection
 // (operand slot (q, j) of step i = column 128c + 32q + 8i + j; proj_down is stored in that order).
@@ -36,17 +38,20 @@ struct QuantParams {
     int M, M_pad, K, R;
 };
 
-constexpr int NW = 8;  // waves per workgroup
+constexpr uint32_t RSRC_WORD3 = 0x00020000;  // raw buffer, 32-bit data format
 
-template <int MT, int RT_MAX, bool FP4>
+// SMOOTH: 0 = no smoothing factors, 1 = the K reciprocal factors are copied to LDS once per workgroup,
+// 2 = read from global memory per chunk (K too large for LDS).
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH>
 __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams p) {
-    extern __shared__ float red[];  // [NW waves][MT][RT][64][4]
+    extern __shared__ float lds[];  // smoothing factors [K] during the walk, then [NW waves][MT][RT][64][4] partial projections
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, q = lane >> 4;
     const int row0 = blockIdx.x * (16 * MT);
     const int kgroups = p.K / 64;
     const int RT = p.R / 16;
+    const int nchunks = p.K / 128;
 
     float4_t acc[MT][RT_MAX];
 #pragma unroll
@@ -54,54 +59,64 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
 #pragma unroll
         for (int rt = 0; rt < RT_MAX; rt++) acc[mt][rt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
+    // The workgroup's rows as a buffer whose size ends with the last valid row: rows beyond M read as zero
+    // without a branch.
+    int rows_valid = p.M - row0;
+    rows_valid = rows_valid < 0 ? 0 : (rows_valid > 16 * MT ? 16 * MT : rows_valid);
+    // (descriptor words made scalar explicitly: a descriptor the compiler takes for lane-dependent is
+    // looped over lane by lane)
+    const uint64_t xbase = (uint64_t)(p.x + (size_t)row0 * p.K);
+    const uint64_t xbase_s = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(xbase >> 32)) << 32) |
+                             (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)xbase);
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)xbase_s, 0, __builtin_amdgcn_readfirstlane(rows_valid * p.K * 2), RSRC_WORD3);
+    const uint32_t x_voff = (uint32_t)(r * p.K + 32 * q) * 2;
+
     // x of one chunk: MT tiles x 4 steps x 8 bf16 per lane
+    // Requests are unconditional (a request behind a branch makes the compiler's wait counting assume the
+    // worst on every path and wait for the chunks requested ahead): a chunk index past the end gets a lane
+    // offset beyond the buffer size instead, which reads zeros and touches no memory.  (The hardware checks
+    // the lane offset against the size, not the scalar offset that carries the chunk.)
     auto load_x = [&](int c, u32x4_t (&xv)[MT][4]) {
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            const int row = row0 + 16 * mt + r;
-            const u32x4_t *src = (const u32x4_t *)(p.x + (size_t)row * p.K + 128 * c + 32 * q);
-#pragma unroll
-            for (int i = 0; i < 4; i++) xv[mt][i] = row < p.M ? src[i] : u32x4_t{0, 0, 0, 0};
-        }
-    };
-    const int nchunks = p.K / 128;
-    u32x4_t xv_next[MT][4];
-    if (wave < nchunks) load_x(wave, xv_next);
-    for (int c = wave; c < nchunks; c += NW) {
-        const int kbase = 128 * c + 32 * q;
-        u32x4_t xv[MT][4];
+        const uint32_t beyond = c < nchunks ? 0u : 0x80000000u;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) xv[mt][i] = xv_next[mt][i];
-        if (c + NW < nchunks) load_x(c + NW, xv_next);
-        // ---- reciprocal smoothing factors of my 32 columns
-        float rs[32];
-        if (p.smooth_rcp) {
-            const float4_t *sp = (const float4_t *)(p.smooth_rcp + kbase);
+            for (int i = 0; i < 4; i++)
+                xv[mt][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (x_voff | beyond) + (uint32_t)(16 * mt * p.K) * 2 + 16 * i, c * 256, 0);
+    };
+    // proj_down as a buffer too: empty when there is no low-rank branch, so that its requests need no branch
+    const __amdgpu_buffer_rsrc_t drsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.down, 0, RT > 0 ? p.K * p.R * 2 : 0, RSRC_WORD3);
+    auto load_down = [&](int c, int i, int rt) {
+        return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(drsrc, lane * 16, (((c * 4 + i) * RT + (rt < RT ? rt : 0)) * 64) * 16, 0));
+    };
+
+    // DEPTH chunks are requested ahead of the one being worked on
+    u32x4_t xv[DEPTH + 1][MT][4];
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                float4_t v = sp[i];
-                rs[4 * i] = v[0]; rs[4 * i + 1] = v[1]; rs[4 * i + 2] = v[2]; rs[4 * i + 3] = v[3];
-            }
+    for (int s = 0; s < DEPTH; s++) load_x(wave + s * NW, xv[s]);
+
+    if (SMOOTH == 1) {
+        for (int k = threadIdx.x * 4; k < p.K; k += 64 * NW * 4) *(float4_t *)&lds[k] = *(const float4_t *)(p.smooth_rcp + k);
+        __syncthreads();
+    }
+
+    auto process = [&](int c, u32x4_t (&x)[MT][4], u32x4_t (&x_ahead)[MT][4]) {
+        const int kbase = 128 * c + 32 * q;
+        // ---- requests first: the low-rank operands of this chunk (all four steps when they fit the
+        // registers), then the activations DEPTH chunks ahead.  In this order a wait for the operands
+        // does not wait for the activations.
+        constexpr bool DOWN_UPFRONT = RT_MAX <= 2;
+        bf16x8_t dn[DOWN_UPFRONT ? 4 : 1][RT_MAX];
+        if (DOWN_UPFRONT) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int rt = 0; rt < RT_MAX; rt++) dn[i][rt] = load_down(c, i, rt);
         }
-        // ---- low-rank down projection on the raw activations
-        if (RT > 0) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-#pragma unroll
-                for (int rt = 0; rt < RT_MAX; rt++) {
-                    if (rt < RT) {
-                        const bf16x8_t b = p.down[((size_t)(c * 4 + i) * RT + rt) * 64 + lane];
-#pragma unroll
-                        for (int mt = 0; mt < MT; mt++) {
-                            bf16x8_t a = __builtin_bit_cast(bf16x8_t, xv[mt][i]);
-                            acc[mt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt][rt], 0, 0, 0);
-                        }
-                    }
-                }
-            }
-        }
+        load_x(c + DEPTH * NW, x_ahead);
+        __builtin_amdgcn_sched_barrier(0);
+
         // ---- smooth, quantize, store
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
@@ -109,13 +124,29 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
             float y[32];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
+                float4_t rs0, rs1;
+                if (SMOOTH == 1) {
+                    rs0 = *(const float4_t *)&lds[kbase + 8 * i];
+                    rs1 = *(const float4_t *)&lds[kbase + 8 * i + 4];
+                } else if (SMOOTH == 2) {
+                    rs0 = *(const float4_t *)(p.smooth_rcp + kbase + 8 * i);
+                    rs1 = *(const float4_t *)(p.smooth_rcp + kbase + 8 * i + 4);
+                }
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const uint32_t w = xv[mt][i][j];
+                    const uint32_t w = x[mt][i][j];
                     const float lo = bits_f32(w << 16), hi = bits_f32(w & 0xFFFF0000u);
                     const int e = 8 * i + 2 * j;
-                    y[e] = p.smooth_rcp ? smooth_quotient(lo, rs[e]) : lo;
-                    y[e + 1] = p.smooth_rcp ? smooth_quotient(hi, rs[e + 1]) : hi;
+                    if (SMOOTH) {
+                        // bf16(x / smooth) for the pair: two products, one packed hardware rounding
+                        const float r0 = j < 2 ? rs0[2 * j] : rs1[2 * j - 4], r1 = j < 2 ? rs0[2 * j + 1] : rs1[2 * j - 3];
+                        const uint32_t pr = pack_bf16x2(__fmul_rn(lo, r0), __fmul_rn(hi, r1));
+                        y[e] = bits_f32(pr << 16);
+                        y[e + 1] = bits_f32(pr & 0xFFFF0000u);
+                    } else {
+                        y[e] = lo;
+                        y[e + 1] = hi;
+                    }
                 }
             }
             const size_t tile = (size_t)(row / 32) * kgroups + (2 * c + (q >> 1));
@@ -124,8 +155,8 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
             if (!FP4) {
                 float s;
                 quantize_int4_half_group<false>(y, 16, words, s);
-                if ((q & 1) == 0)
-                    ((uint16_t *)p.oscales)[(size_t)(2 * c + (q >> 1)) * p.M_pad + row] = (uint16_t)f32_to_bf16_bits(s);
+                // (both lanes of a group hold the same scale and store it: no branch)
+                ((uint16_t *)p.oscales)[(size_t)(2 * c + (q >> 1)) * p.M_pad + row] = (uint16_t)f32_to_bf16_bits(s);
             } else {
                 uint32_t sc[2];
                 quantize_nvfp4_two_groups(y, words, sc);
@@ -135,15 +166,39 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
             }
             *(u32x4_t *)dst = words;
         }
+
+        // ---- low-rank down projection on the raw activations (rank tiles beyond R repeat tile 0 into
+        // accumulators that are never stored: cheaper than a branch per tile)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int rt = 0; rt < RT_MAX; rt++) {
+                const bf16x8_t b = DOWN_UPFRONT ? dn[i][rt] : load_down(c, i, rt);
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++)
+                    acc[mt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, x[mt][i]), b, acc[mt][rt], 0, 0, 0);
+            }
+    };
+
+    // wave w walks the chunks w, w + NW, ...; the ring of DEPTH + 1 register buffers is indexed statically
+    for (int c0 = wave;; c0 += (DEPTH + 1) * NW) {
+#pragma unroll
+        for (int s = 0; s <= DEPTH; s++) {
+            const int c = c0 + s * NW;
+            if (c >= nchunks) goto walked;
+            process(c, xv[s], xv[(s + DEPTH) % (DEPTH + 1)]);
+        }
     }
+walked:
 
     // ---- reduce the waves' partial projections and write lora_act[row][rank]
     if (RT > 0) {
+        if (SMOOTH == 1) __syncthreads();  // the factors in LDS are not needed any more
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int rt = 0; rt < RT_MAX; rt++)
-                if (rt < RT) *(float4_t *)&red[(((wave * MT + mt) * RT + rt) * 64 + lane) * 4] = acc[mt][rt];
+                if (rt < RT) *(float4_t *)&lds[(((wave * MT + mt) * RT + rt) * 64 + lane) * 4] = acc[mt][rt];
         __syncthreads();
         const int total = 16 * MT * p.R;
         for (int idx = threadIdx.x; idx < total; idx += 64 * NW) {
@@ -152,16 +207,19 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
             const int src_lane = 16 * (rr / 4) + rc, i = rr % 4;  // 16x16 MFMA result layout
             float sum = 0.f;
 #pragma unroll
-            for (int w = 0; w < NW; w++) sum += red[(((w * MT + mt) * RT + rt) * 64 + src_lane) * 4 + i];
+            for (int w = 0; w < NW; w++) sum += lds[(((w * MT + mt) * RT + rt) * 64 + src_lane) * 4 + i];
             p.lora_out[(size_t)(row0 + row) * p.R + rank] = sum;
         }
     }
 }
 
-template <int MT, int RT_MAX, bool FP4>
-int launch(const QuantParams &p, hipStream_t stream) {
-    const size_t smem = (size_t)NW * MT * (p.R / 16) * 64 * 4 * sizeof(float);
-    auto kern = quantize_fuse_lora_kernel<MT, RT_MAX, FP4>;
+constexpr size_t SMOOTH_LDS_MAX = 64 * 1024;  // two workgroups of a compute unit must fit side by side
+
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH>
+int launch_as(const QuantParams &p, hipStream_t stream) {
+    size_t smem = (size_t)NW * MT * (p.R / 16) * 64 * 4 * sizeof(float);
+    if (SMOOTH == 1 && (size_t)p.K * 4 > smem) smem = (size_t)p.K * 4;
+    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH>;
     if (smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "quantize: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
@@ -170,13 +228,22 @@ int launch(const QuantParams &p, hipStream_t stream) {
     return check_launch("quantize_w4a4_act_fuse_lora");
 }
 
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4>
+int launch(const QuantParams &p, hipStream_t stream) {
+    if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0>(p, stream);
+    if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1>(p, stream);
+    return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2>(p, stream);
+}
+
 template <bool FP4>
 int dispatch(const QuantParams &p, hipStream_t stream) {
-    // rows per workgroup: enough workgroups to cover the chip, but amortise proj_down reads at high rank
+    // Rows per workgroup: 16 while that gives the chip enough workgroups, 32 to amortise the proj_down
+    // reads at high rank.  Four waves of up to 256 registers: two workgroups fit a compute unit, so that a
+    // workgroup count a little above the number of compute units does not cost a second round.
     const int RT = p.R / 16;
-    if (RT <= 2) return p.M_pad >= 8192 ? launch<2, 2, FP4>(p, stream) : launch<1, 2, FP4>(p, stream);
-    if (RT <= 4) return launch<2, 4, FP4>(p, stream);
-    if (RT <= 8) return launch<2, 8, FP4>(p, stream);
+    if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4>(p, stream) : launch<4, 1, 2, 2, FP4>(p, stream);
+    if (RT <= 4) return launch<4, 2, 4, 1, FP4>(p, stream);
+    if (RT <= 8) return launch<4, 2, 8, 1, FP4>(p, stream);
     return fail(SVDQ_EUNSUPPORTED, "quantize: rank %d > 128 is not supported", p.R);
 }
 
@@ -190,7 +257,7 @@ extern "C" int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *a, voi
     SVDQ_REQUIRE(a->K > 0 && a->K % 128 == 0, "quantize: K (%lld) must be a multiple of 128", (long long)a->K);
     SVDQ_REQUIRE(a->R >= 0 && a->R % 16 == 0, "quantize: rank (%lld) must be a multiple of 16", (long long)a->R);
     SVDQ_REQUIRE(a->R == 0 || (a->lora_down && a->lora_act_out), "quantize: lora_down/lora_act_out must be given when R > 0");
-    SVDQ_REQUIRE(a->M_pad < (1ll << 31) / 4 && a->K < (1 << 24), "quantize: shape too large");
+    SVDQ_REQUIRE(a->M_pad < (1ll << 31) / 4 && a->K < (1 << 24) && a->K * a->R < (1ll << 30), "quantize: shape too large");
     SVDQ_REQUIRE(((uintptr_t)a->input % 16 == 0) && ((uintptr_t)a->output % 16 == 0) && ((uintptr_t)a->lora_down % 16 == 0) &&
                      ((uintptr_t)a->smooth_rcp % 16 == 0),
                  "quantize: pointers must be 16-byte aligned");

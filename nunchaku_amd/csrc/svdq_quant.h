@@ -22,12 +22,18 @@ __device__ inline float smooth_quotient(float x, float rcp) {
     return bf16_bits_to_f32(f32_to_bf16_bits(__fmul_rn(x, rcp)));
 }
 
-// 8 clamped-and-rounded codes (already offset so that they are in [0, 15]) -> one word
+// 8 clamped-and-rounded codes (already offset so that they are in [0, 15]) -> one word.  Every input is
+// RNE_MAGIC + u, bit pattern 0x4B400000 | u: bits [21:4] are zero, so four of them chain into 16 clean
+// low bits with shift-and-or alone (the constant's bits stay at or above bit 22), and one byte
+// permute joins the two halves: 7 instructions per word.
 __device__ inline uint32_t pack8(const float (&v)[8]) {
-    uint32_t w = 0;
+    uint32_t lo = f32_bits(v[3]), hi = f32_bits(v[7]);
 #pragma unroll
-    for (int j = 0; j < 8; j++) w |= (f32_bits(v[j]) & 15u) << (4 * j);
-    return w;
+    for (int j = 2; j >= 0; j--) {
+        lo = (lo << 4) | f32_bits(v[j]);
+        hi = (hi << 4) | f32_bits(v[4 + j]);
+    }
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes 0, 1 of lo below bytes 0, 1 of hi
 }
 
 // fp32 (finite, >= 0, <= 448) -> e4m3 bit pattern, round to nearest even
