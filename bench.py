@@ -90,6 +90,9 @@ def main():
     ap.add_argument("--workload", default="flux_mlp_fc1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=4608)
+    ap.add_argument("--qkv-rope", action="store_true",
+                    help="time the GEMM with the RMS-norm + rotary epilogue of fused_qkv_norm_rottary (workload flux_qkv); "
+                         "the CPU comparison is skipped")
     ap.add_argument("--only", choices=["gemm", "quantize", "copy", "mfma-rate"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
                          "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters; "
@@ -134,9 +137,29 @@ def main():
     t = mod.native_tensors()
     from nunchaku_amd.ops import svdq_quantize_w4a4_act_fuse_lora
 
+    gemm = lambda: mod.forward_quant(qx, asc, la, out)  # noqa: E731
+    if args.qkv_rope:
+        if N % 384 != 0:
+            sys.exit("--qkv-rope needs a QKV-shaped workload (N three equal parts of 128-wide heads): use --workload flux_qkv")
+        from nunchaku_amd import packing
+        from nunchaku_amd.ops import svdq_gemm_w4a4
+
+        args.no_cpu = True
+        gen = torch.Generator().manual_seed(cfg["seed"])
+        ang = torch.rand(M_pad, 64, generator=gen) * 6.283
+        # (sin, cos) pairs stay adjacent in the reference's packed order, so a table of random angles is as
+        # good a packed table as any: taken as written by pack_rotemb and converted like a caller's table
+        rot = packing.repack_rotemb(torch.stack((torch.sin(ang), torch.cos(ang)), dim=-1).reshape(M_pad, 128).to(dev))
+        nq = (1.0 + 0.2 * torch.randn(128, generator=gen)).to(torch.bfloat16).to(dev)
+        nk = (1.0 + 0.2 * torch.randn(128, generator=gen)).to(torch.bfloat16).to(dev)
+
+        def gemm():
+            svdq_gemm_w4a4(act=qx, wgt=t["qweight"], out=out, ascales=asc, wscales=t["wscales"], lora_act_in=la,
+                           lora_up=t["proj_up"], bias=t["bias"], norm_q=nq, norm_k=nk, rotary_emb=rot)
+
     def step():
         svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
-        mod.forward_quant(qx, asc, la, out)
+        gemm()
 
     if args.only:
         svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
@@ -144,7 +167,7 @@ def main():
         t0 = time.perf_counter()
         for _ in range(args.steps):
             if args.only == "gemm":
-                mod.forward_quant(qx, asc, la, out)
+                gemm()
             else:
                 svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
         torch.cuda.synchronize()
@@ -167,7 +190,7 @@ def main():
         e[0].record()
         svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
         e[1].record()
-        mod.forward_quant(qx, asc, la, out)
+        gemm()
         e[2].record()
     torch.cuda.synchronize()
     tq_us = statistics.mean(e[0].elapsed_time(e[1]) for e in evs) * 1e3
@@ -183,7 +206,8 @@ def main():
         "value": value, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: SVDQW4A4Linear forward M={M} K={K} N={N} rank={R} INT4 g64 bf16 in/out",
+        "config": {"workload": f"{args.workload}: SVDQW4A4Linear forward M={M} K={K} N={N} rank={R} INT4 g64 bf16 in/out"
+                               + (" + RMS norm and rotary embedding on q, k in the GEMM epilogue" if args.qkv_rope else ""),
                    "M": M, "K": K, "N": N, "rank": R},
         "pct_of_int8_mfma_peak": 100.0 * value / INT8_PEAK_TOPS,
         "us_per_layer": ms_per_step * 1e3,
@@ -194,7 +218,7 @@ def main():
             "gemm_main_term_TOPS": 2.0 * M * N * K / (tg_us * 1e-6) / 1e12,
         },
         "roofline": {
-            "kernel": "gemm_w4a4_kernel<false, false, false>", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
+            "kernel": "gemm_w4a4_kernel<false, false, true>" if args.qkv_rope else "gemm_w4a4_kernel<false, false, false>", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
             "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": PROFILED_GEMM_TRAFFIC_BYTES.get(args.workload),
             "peak_basis": "dense INT8 MFMA (the metric's peak); the kernel issues fp16 MFMA, dense peak 2500",
             "frac_of_fp16_mfma_peak": gemm_tops / FP16_PEAK_TFLOPS,

@@ -32,7 +32,7 @@ extern "C" {
 #define SVDQ_EUNSUPPORTED -2 /* valid request that this build does not implement */
 #define SVDQ_ELAUNCH -3      /* the HIP runtime refused the launch */
 
-#define SVDQ_ABI_VERSION 1
+#define SVDQ_ABI_VERSION 2
 
 int svdq_abi_version(void);
 const char *svdq_last_error(void);
@@ -77,6 +77,12 @@ int svdq_repack_lora_down(const void *src, void *dst, int64_t K, int64_t R, void
 
 /* proj_up bf16 [N, R] (reference lane order) -> bf16 [N, R] row-major in channel/rank order. */
 int svdq_repack_lora_up(const void *src, void *dst, int64_t N, int64_t R, void *stream);
+
+/* Rotary table fp32 [rows, 128] in the order written by pack_rotemb (nunchaku/models/embeddings.py:88-120:
+ * per 16 rows and 8 floats the fp32 accumulator fragment of an m16n8 MMA; loaded by
+ * EpilogueRMSNormRope::load_rotemb, src/kernels/zgemm/epilogues.cuh:282-305) -> the order the GEMM
+ * epilogue reads, [rows/32][16][64][4] (see svdq_gemm_args.rotary_emb).  rows: a multiple of 32. */
+int svdq_repack_rotemb(const void *src, void *dst, int64_t rows, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Operator 1: smooth + quantize activations + low-rank down projection, one pass over x.
@@ -146,6 +152,20 @@ typedef struct svdq_gemm_args {
     int32_t act_unsigned;   /* INT4 activations are unsigned codes 0..15                            */
     int32_t fuse_silu;      /* must be 0 (not implemented)                                          */
     int32_t fp4;            /* operands are NVFP4                                                   */
+    /* RMS norm + rotary embedding of the q and k thirds of a fused QKV projection (all NULL / 0
+     * otherwise).  Replaces EpilogueRMSNormRope, src/kernels/zgemm/epilogues.cuh:269-425, composed as in
+     * gemm_w4a4_launch_impl.cuh:347-402 (after bias and low-rank up, before the store).  Columns
+     * [0, N/3) are q, [N/3, 2N/3) are k, the rest (v) passes through; heads are 128 columns wide;
+     * N must be a multiple of 384.  Per row and head: x *= rsqrt(mean(x^2) + norm_eps) * weight, then
+     * every pair (x[2i], x[2i+1]) is rotated by (sin, cos) = rotary_emb[row][2i], [2i+1].          */
+    const void *norm_q;     /* bf16 [128]                                                           */
+    const void *norm_k;     /* bf16 [128]                                                           */
+    const float *rotary_emb;/* fp32, rot_rows * 128 values in the order [rot_rows/32][16][64][4]: block b,
+                               slot s = 4 nt + q, lane l = r + 32 h hold floats 32 nt + 8 q + 4 h + [0, 4)
+                               of row 32 b + r, where float 2i of a row is sin and 2i + 1 cos of pair i
+                               (svdq_repack_rotemb writes it from the reference's pack_rotemb order)  */
+    int64_t rot_rows;       /* rows of rotary_emb: M_out <= rot_rows <= M_pad, a multiple of 32      */
+    float norm_eps;         /* the reference uses 1e-6 (launch_impl.cuh:374)                        */
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);

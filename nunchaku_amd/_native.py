@@ -25,11 +25,11 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
-SVDQ_ABI_VERSION = 1
+SVDQ_ABI_VERSION = 2
 EXPORTED_SYMBOLS = [
     "svdq_abi_version", "svdq_last_error",
     "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
-    "svdq_repack_smooth", "svdq_repack_lora_down", "svdq_repack_lora_up",
+    "svdq_repack_smooth", "svdq_repack_lora_down", "svdq_repack_lora_up", "svdq_repack_rotemb",
     "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4",
 ]
 
@@ -60,6 +60,8 @@ class GemmArgs(ctypes.Structure):
         ("R_up", ctypes.c_int64), ("R_down", ctypes.c_int64),
         ("alpha", ctypes.c_float), ("act_unsigned", ctypes.c_int32), ("fuse_silu", ctypes.c_int32),
         ("fp4", ctypes.c_int32),
+        ("norm_q", ctypes.c_void_p), ("norm_k", ctypes.c_void_p), ("rotary_emb", ctypes.c_void_p),
+        ("rot_rows", ctypes.c_int64), ("norm_eps", ctypes.c_float),
     ]
 
 
@@ -125,6 +127,7 @@ def lib() -> ctypes.CDLL:
         L.svdq_repack_smooth.argtypes = [vp, vp, i64, vp]
         L.svdq_repack_lora_down.argtypes = [vp, vp, i64, i64, vp]
         L.svdq_repack_lora_up.argtypes = [vp, vp, i64, i64, vp]
+        L.svdq_repack_rotemb.argtypes = [vp, vp, i64, vp]
         L.svdq_quantize_w4a4_act_fuse_lora.argtypes = [ctypes.POINTER(QuantizeArgs), vp]
         L.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), vp]
         for name in EXPORTED_SYMBOLS:

@@ -114,6 +114,18 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
 #endif
     SVDQ_REQUIRE(a->R_down >= 0 && a->R_down % 16 == 0 && a->R_down <= 128, "gemm: R_down (%lld) must be a multiple of 16, at most 128", (long long)a->R_down);
 
+    if (a->rotary_emb) {
+        SVDQ_REQUIRE(a->norm_q && a->norm_k, "gemm: rotary_emb needs norm_q and norm_k");
+        SVDQ_REQUIRE(a->N % 384 == 0, "gemm: rotary_emb needs N (%lld) to be three equal parts of 128-wide heads", (long long)a->N);
+        SVDQ_REQUIRE(a->out && !a->qout && a->N_out == a->N, "gemm: rotary_emb goes with a full-width `out` and no qout");
+        SVDQ_REQUIRE(a->rot_rows >= a->M_out && a->rot_rows <= a->M_pad && a->rot_rows % 32 == 0,
+                     "gemm: rotary_emb has %lld rows for %lld output rows (must cover them, in whole blocks of 32)", (long long)a->rot_rows, (long long)a->M_out);
+        SVDQ_REQUIRE(((uintptr_t)a->rotary_emb % 16 == 0) && ((uintptr_t)a->norm_q % 8 == 0) && ((uintptr_t)a->norm_k % 8 == 0),
+                     "gemm: rotary_emb / norm pointers are not aligned");
+    } else {
+        SVDQ_REQUIRE(!a->norm_q && !a->norm_k, "gemm: norm_q / norm_k need rotary_emb");
+    }
+
     GemmParams p;
 #ifdef SVDQ_GEMM_TIMING
     p.stamps = (long long *)a->next_lora_act_out;  // debug builds borrow this slot for the stamp buffer
@@ -140,6 +152,12 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     p.M_out = (int)a->M_out; p.N_out = (int)a->N_out; p.R_up = (int)a->R_up;
     p.alpha = a->alpha;
     for (int i = 0; i < 8; i++) p.lora_scales[i] = (a->lora_scales && i < (a->R_up + 15) / 16) ? a->lora_scales[i] : 1.0f;
+    p.norm_q = (const uint16_t *)a->norm_q;
+    p.norm_k = (const uint16_t *)a->norm_k;
+    p.rotary = a->rotary_emb;
+    p.rot_rows = (int)a->rot_rows;
+    p.rope_cols = (int)(a->N / 3 * 2);
+    p.norm_eps = a->norm_eps;
     p.gelu = a->qout != nullptr;  // the GELU is composed exactly when the next layer's input is produced (launch_impl.cuh:282-309)
 #ifdef SVDQ_GEMM_TIMING
     p.next_down = nullptr; p.next_lora_out = nullptr; p.R_down = 0;
@@ -171,7 +189,8 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
         p.counters = (int *)w->ptr;
         p.partials = (float *)(w->ptr + w->counters_bytes);
     }
-    const bool next = a->qout != nullptr || a->next_lora_down != nullptr;
+    // (the kernels with the next-layer epilogue also carry the norm + rotary epilogue)
+    const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr;
     if (p.next_lora_out) {  // the low-rank projection for the next layer is accumulated across column blocks
         const int64_t n = a->M_pad * a->R_down;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, p.next_lora_out, n);

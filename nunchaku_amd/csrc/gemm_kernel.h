@@ -115,6 +115,9 @@ __device__ inline float4_t load_partial(__amdgpu_buffer_rsrc_t r, int tid, int q
 
 // NEXT: the epilogue also prepares the next layer's input (GELU, quantize, low-rank down); the plain
 // variant carries none of that code or of its registers.
+#ifndef SVDQ_ROPE_ENABLED
+#define SVDQ_ROPE_ENABLED true
+#endif
 template <bool ACT_UNSIGNED, bool FP4, bool NEXT>
 __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -629,6 +632,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
             coltab[2 * lane + j] = cf;
             coltab[128 + 2 * lane + j] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+            if (NEXT && p.rotary)  // RMS-norm weights of the head these 128 columns are (q below N/3, k below 2N/3)
+                ((float *)(lds + NORMW_OFF + wave * 512))[2 * lane + j] = bf16_bits_to_f32((wcol0 < p.rope_cols / 2 ? p.norm_q : p.norm_k)[2 * lane + j]);
         }
     }
     // Low-rank up projection (lora.cuh:110-241): out += bf16(lora_act * scale) @ up^T on the matrix cores.
@@ -810,6 +815,48 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #pragma unroll
                 for (int nt = 0; nt < 4; nt++)
                     v[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_lb(nt, s2), la, v[nt], 0, 0, 0);
+            }
+        }
+        if (NEXT && SVDQ_ROPE_ENABLED && p.rotary && wcol0 < p.rope_cols) {
+            // EpilogueRMSNormRope (epilogues.cuh:269-425): the wave's 128 columns are one head of q or k.
+            // The lane holds 64 values of its row, lane ^ 32 the other 64.  The (sin, cos) table is stored in
+            // this loop's order ([32-row block][nt][q][lane] x float4: a wave-wide request is 1 KB
+            // contiguous), requested two column tiles ahead.
+            int blk = (wrow0 + mt * 32) >> 5;
+            blk = blk < (p.rot_rows >> 5) ? blk : (p.rot_rows >> 5) - 1;  // (rows beyond the output are never stored)
+            const float4_t *rp = (const float4_t *)p.rotary + (size_t)blk * (16 * 64) + lane;
+            const float *normw = (const float *)(lds + NORMW_OFF + wave * 512);
+            float4_t sc[2][4];
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) sc[nt][q] = rp[(nt * 4 + q) * 64];
+            float ss = 0.f;
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) ss += v[nt][e] * v[nt][e];
+            ss += __shfl_xor(ss, 32);
+            const float coef = __builtin_amdgcn_rsqf(ss * (1.0f / 128.0f) + p.norm_eps);
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4_t w4 = *(const float4_t *)(normw + nt * 32 + 8 * q + 4 * h);
+                    const float4_t s4 = sc[nt & 1][q];  // sin, cos of the two pairs
+#pragma unroll
+                    for (int pr = 0; pr < 2; pr++) {
+                        const float x = v[nt][4 * q + 2 * pr] * (coef * w4[2 * pr]);
+                        const float y = v[nt][4 * q + 2 * pr + 1] * (coef * w4[2 * pr + 1]);
+                        const float sn = s4[2 * pr], cs = s4[2 * pr + 1];
+                        v[nt][4 * q + 2 * pr] = x * cs - y * sn;
+                        v[nt][4 * q + 2 * pr + 1] = x * sn + y * cs;
+                    }
+                }
+                if (nt < 2) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) sc[nt & 1][q] = rp[((nt + 2) * 4 + q) * 64];
+                }
             }
         }
         if (NEXT && p.gelu) {

@@ -20,7 +20,8 @@ constexpr int SLAB_OFF = STAGES * STAGE_BYTES;     // 4 waves x (32 rows x OUT_L
 constexpr int SHIFT_OFF = SLAB_OFF + 4 * 32 * OUT_LD * 2;  // int [MAX_BATCH][256] row renormalisation shifts
 constexpr int TAB_OFF = SHIFT_OFF + MAX_BATCH * 256 * 4;   // 4 waves x float [2][128]: column factors and biases
 constexpr int FLAG_OFF = TAB_OFF + 4 * 1024;               // one word: a thread's reading of an arrival counter, for all
-constexpr int LDS_BYTES = FLAG_OFF + 16;
+constexpr int NORMW_OFF = FLAG_OFF + 16;                   // 4 waves x float [128]: RMS-norm weights of the wave's head
+constexpr int LDS_BYTES = NORMW_OFF + 4 * 512;
 constexpr int NORM_TARGET_EXP = 10;
 
 
@@ -50,6 +51,11 @@ struct GemmParams {
     float alpha;
     float lora_scales[8];
     int gelu;
+    // RMS norm + rotary embedding on the q and k heads of a fused QKV projection (next-layer variants only)
+    const uint16_t *norm_q, *norm_k;  // bf16 [128]
+    const float *rotary;              // fp32 [rot_rows/32][16][64 lanes][4], see svdq_gemm_args; null: no such epilogue
+    int rot_rows, rope_cols;          // rope_cols = 2 N / 3: the columns of q and k
+    float norm_eps;
 };
 
 

@@ -156,6 +156,22 @@ __global__ void repack_lora_up_kernel(const uint16_t *__restrict__ src, uint16_t
     dst[i] = src[lora_src_index(i / R, i % R, R, false)];
 }
 
+// Rotary table: one thread per float of the native order [rows/32][16 slots][64 lanes][4].  Source: the
+// order written by pack_rotemb (nunchaku/models/embeddings.py:88-120) = float4 [rows/16][16 tiles j][32
+// lanes], lane 4 g + t holding floats 8 j + 2 t + {0, 1} of rows g (.xy) and g + 8 (.zw)
+// (loader: src/kernels/zgemm/epilogues.cuh:282-305).
+__global__ void repack_rotemb_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows) {
+    const int64_t o = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+    if (o >= rows * 128) return;
+    const int e = (int)(o & 3), l = (int)((o >> 2) & 63), s = (int)((o >> 8) & 15);
+    const int64_t b = o >> 12;
+    const int64_t row = 32 * b + (l & 31);
+    const int d = 32 * (s >> 2) + 8 * (s & 3) + 4 * (l >> 5) + e;  // float of the row: sin of pair d/2 (even d) or cos (odd d)
+    const int rr = (int)(row & 15), g = rr & 7, half = rr >> 3;
+    const int j = d >> 3, t = (d & 7) >> 1;
+    dst[o] = src[((((row >> 4) * 16 + j) * 8 + g) * 4 + t) * 4 + half * 2 + (d & 1)];
+}
+
 inline unsigned blocks_for(int64_t n, int bs = 256) { return (unsigned)((n + bs - 1) / bs); }
 
 }  // namespace
@@ -224,6 +240,14 @@ int svdq_repack_lora_up(const void *src, void *dst, int64_t N, int64_t R, void *
     hipLaunchKernelGGL(repack_lora_up_kernel, dim3(blocks_for(N * R)), dim3(256), 0, (hipStream_t)stream,
                        (const uint16_t *)src, (uint16_t *)dst, N, R);
     return check_launch("repack_lora_up");
+}
+
+int svdq_repack_rotemb(const void *src, void *dst, int64_t rows, void *stream) {
+    SVDQ_REQUIRE(src && dst && src != dst, "repack_rotemb: null or aliased pointer");
+    SVDQ_REQUIRE(rows > 0 && rows % 32 == 0, "repack_rotemb: rows (%lld) must be a positive multiple of 32", (long long)rows);
+    hipLaunchKernelGGL(repack_rotemb_kernel, dim3(blocks_for(rows * 128)), dim3(256), 0, (hipStream_t)stream, (const float *)src,
+                       (float *)dst, rows);
+    return check_launch("repack_rotemb");
 }
 
 }  // extern "C"

@@ -1,6 +1,6 @@
 """Operator wrappers with the signatures of ``nunchaku.ops`` (nunchaku/ops/{quantize,gemm,fused}.py)."""
 
-from .fused import fused_gelu_mlp
+from .fused import fused_gelu_mlp, fused_qkv_norm_rottary
 from .gemm import svdq_gemm_w4a4, svdq_gemm_w4a4_cuda
 from .quantize import svdq_quantize_w4a4_act_fuse_lora, svdq_quantize_w4a4_act_fuse_lora_cuda
 
@@ -10,4 +10,5 @@ __all__ = [
     "svdq_gemm_w4a4",
     "svdq_gemm_w4a4_cuda",
     "fused_gelu_mlp",
+    "fused_qkv_norm_rottary",
 ]

@@ -12,7 +12,8 @@ import torch
 from .. import _native as nv
 from .. import packing
 
-_NOT_BUILT = ("poolout", "norm_q", "norm_k", "rotary_emb", "out_vk", "out_linearattn", "out_q", "out_k", "out_v")
+_NOT_BUILT = ("poolout", "out_vk", "out_linearattn", "out_q", "out_k", "out_v")
+NORM_EPS = 1e-6  # gemm_w4a4_launch_impl.cuh:374
 
 
 def svdq_gemm_w4a4(
@@ -52,7 +53,10 @@ def svdq_gemm_w4a4(
     wgt / wscales / lora_up / bias / wcscales / smooth_factor / lora_down: the layer's tensors, in
     the reference checkpoint layout (repacked once and cached) or already native (``packing``);
     out      bf16 [M, N] (M <= M_pad);  qout / oscales / lora_act_out: inputs of the next layer, in
-    which case a tanh-GELU is applied first (gemm_w4a4_launch_impl.cuh:282-309).
+    which case a tanh-GELU is applied first (gemm_w4a4_launch_impl.cuh:282-309);
+    norm_q / norm_k bf16 [128] and rotary_emb fp32 [B, M/B, 128] (packed by ``pack_rotemb``): RMS norm
+    and rotary embedding on the q and k thirds of ``out`` (launch_impl.cuh:347-402, the ``out`` form;
+    the ``out_q / out_k / out_v`` form that packs for the attention kernel is not built).
     """
     local = locals()
     for name in _NOT_BUILT:
@@ -70,6 +74,10 @@ def svdq_gemm_w4a4(
         raise ValueError("one of out / qout is required")
     if qout is not None and (oscales is None or smooth_factor is None):
         raise ValueError("qout needs oscales and smooth_factor")
+    if rotary_emb is not None and (norm_q is None or norm_k is None):
+        raise ValueError("rotary_emb needs norm_q and norm_k")  # the reference asserts both (launch_impl.cuh:348-349)
+    if rotary_emb is None and (norm_q is not None or norm_k is not None):
+        raise ValueError("norm_q / norm_k need rotary_emb")
 
     if lora_up is not None and lora_up.shape[1] == 0:  # rank-0 layer: no low-rank branch
         lora_up = lora_act_in = None
@@ -99,6 +107,16 @@ def svdq_gemm_w4a4(
     if out is not None and out.dtype != torch.bfloat16:
         raise NotImplementedError("only bf16 outputs are supported")
 
+    rot_n = None
+    if rotary_emb is not None:
+        rot_n = packing.native(rotary_emb, "rotemb")
+        for name, t in (("norm_q", norm_q), ("norm_k", norm_k)):
+            nv.require_gpu(t, name)
+            if t.dtype != torch.bfloat16 or t.numel() != 128 or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous bf16 vector of 128 elements (one head)")
+        if out is None or out.shape[-1] != N:
+            raise ValueError("rotary_emb needs a full-width `out`")
+
     n_sc = max(1, math.ceil(rank_up / 16))
     sc = (ctypes.c_float * n_sc)(*[float(lora_scales[i]) if i < len(lora_scales) else 0.0 for i in range(n_sc)])
     M_out = 0 if out is None else out.numel() // out.shape[-1]
@@ -112,6 +130,8 @@ def svdq_gemm_w4a4(
         M_pad=M_pad, N=N, K=K, M_out=M_out, N_out=N_out, R_up=rank_up,
         R_down=0 if lora_down is None else lora_down.shape[1],
         alpha=float(alpha), act_unsigned=int(act_unsigned), fuse_silu=int(fuse_silu), fp4=int(fp4),
+        norm_q=nv.ptr(norm_q), norm_k=nv.ptr(norm_k), rotary_emb=nv.ptr(rot_n),
+        rot_rows=0 if rot_n is None else rot_n.shape[0], norm_eps=NORM_EPS,
     )
     nv.check(nv.lib().svdq_gemm_w4a4(ctypes.byref(args), nv.stream_ptr(dev)))
 

@@ -90,6 +90,21 @@ def repack_lora_up(proj_up: torch.Tensor) -> torch.Tensor:
     return _tag(out, "lora_up")
 
 
+def repack_rotemb(rotemb: torch.Tensor) -> torch.Tensor:
+    """Rotary table fp32 [B, M, 128] (or [M, 128]) in the order written by ``pack_rotemb``
+    (nunchaku/models/embeddings.py:88-120) -> the order the GEMM epilogue reads (same element count;
+    ``include/svdq_amd.h``, ``svdq_gemm_args.rotary_emb``).  The row count must be a multiple of 32."""
+    nv.require_gpu(rotemb, "rotary_emb")
+    if rotemb.dtype != torch.float32 or not rotemb.is_contiguous():
+        raise ValueError("rotary_emb must be a contiguous float32 tensor")
+    rows = rotemb.numel() // rotemb.shape[-1]
+    if rotemb.shape[-1] != 128:
+        raise ValueError(f"rotary_emb must be [.., M, 128], got {tuple(rotemb.shape)}")
+    out = torch.empty(rows, 128, dtype=torch.float32, device=rotemb.device)
+    nv.check(nv.lib().svdq_repack_rotemb(rotemb.data_ptr(), out.data_ptr(), rows, nv.stream_ptr(rotemb.device)))
+    return _tag(out, "rotemb")
+
+
 _REPACKERS = {
     "qweight": repack_qweight,
     "wscales": repack_wscales,
@@ -97,6 +112,7 @@ _REPACKERS = {
     "smooth_rcp": repack_smooth,
     "lora_down": repack_lora_down,
     "lora_up": repack_lora_up,
+    "rotemb": repack_rotemb,
 }
 
 # (data_ptr, version, shape, dtype, kind, fp4) -> (weakref to the source, native tensor)

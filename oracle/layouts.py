@@ -188,3 +188,40 @@ def unpack_lora(stored: np.ndarray, down: bool) -> np.ndarray:
     out = np.zeros((C, R), dtype=stored.dtype)
     out[ch, rk] = stored.reshape(-1)
     return out
+
+
+# --------------------------------------------------------------------------------------------
+# rotary table: logical fp32 [M, D] ((sin, cos) of pair i at [2i], [2i+1])  ->  packed fp32 [M, D]
+# --------------------------------------------------------------------------------------------
+
+
+def pack_rotemb(rotemb: np.ndarray) -> np.ndarray:
+    """pack_rotemb, nunchaku/models/embeddings.py:88-120, for one batch entry: the reshape/permute
+    recipe, written with numpy axes.  ``rotemb``: fp32 [M, D] with M % 16 == 0 and D % 8 == 0."""
+    M, D = rotemb.shape
+    assert M % 16 == 0 and D % 8 == 0
+    r = rotemb.reshape(M // 16, 16, D // 8, 8).transpose(0, 2, 1, 3)      # [M/16][D/8][16 rows][8 floats]
+    r = r.reshape(M // 16, D // 8, 2, 8, 4, 2).transpose(0, 1, 3, 4, 2, 5)  # rows -> (half, g), floats -> (t, s)
+    return np.ascontiguousarray(r).reshape(M, D)
+
+
+def rotemb_index(M: int, D: int):
+    """For every stored float, in storage order, its logical (row, float index), read off the loader
+    EpilogueRMSNormRope::load_rotemb and the use of the loaded float4 in ``apply``
+    (src/kernels/zgemm/epilogues.cuh:282-305,383-401): storage = float4 ``[M/16][D/8][lane:32]``;
+    lane = 4 g + t holds, for the m16n8 accumulator tile j of the head, (sin, cos) of rows g and
+    g + 8 (float4 .xy and .zw) for the pair at columns 8 j + 2 t, 8 j + 2 t + 1."""
+    mb, j, lane, half, s = np.meshgrid(np.arange(M // 16), np.arange(D // 8), np.arange(32), np.arange(2), np.arange(2), indexing="ij")
+    g, t = lane // 4, lane % 4
+    row = 16 * mb + g + 8 * half
+    col = 8 * j + 2 * t + s
+    return row.reshape(-1), col.reshape(-1)
+
+
+def unpack_rotemb(stored: np.ndarray) -> np.ndarray:
+    """Inverse of :func:`pack_rotemb` through the closed form."""
+    M, D = stored.shape
+    row, col = rotemb_index(M, D)
+    out = np.empty_like(stored)
+    out[row, col] = stored.reshape(-1)
+    return out

@@ -128,3 +128,29 @@ def fused_gelu_mlp(x: torch.Tensor, fc1: FakeQuantLinear, fc2: FakeQuantLinear, 
         qcodes, qscales = quant.quantize_act_int4(h.to(torch.bfloat16), fc2.smooth, unsigned=True, shift=quant.SHIFT_GELU)
     out = fc2.forward_quant(qcodes, qscales, lora2, double=double)[: x.shape[0]]
     return out, {"h": h, "qcodes": qcodes, "qscales": qscales, "lora2": lora2}
+
+
+def rmsnorm_rope(out: torch.Tensor, norm_q: torch.Tensor, norm_k: torch.Tensor, rotemb: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """EpilogueRMSNormRope (src/kernels/zgemm/epilogues.cuh:269-425) on the output of a fused QKV
+    projection, composed after bias and low-rank up (gemm_w4a4_launch_impl.cuh:347-402).
+
+    out fp32 [M, N] with N = 3 * heads * 128: columns [0, N/3) are q, [N/3, 2N/3) are k, the rest is
+    v and passes through (epilogues.cuh:413-424).  Per row and 128-wide head:
+    ``x *= rsqrt(mean(x^2) + eps) * weight`` (:338-372), then every pair (x[2i], x[2i+1]) is rotated:
+    ``(x cos - y sin, x sin + y cos)`` with (sin, cos) = rotemb[row, 2i], rotemb[row, 2i + 1]
+    (:374-392; the table is [M, 128] logical, see layouts.pack_rotemb).  Evaluated in fp64; the
+    reference rounds to bf16 before and after, the caller rounds where it stores.
+    """
+    M, N = out.shape
+    assert N % 384 == 0 and rotemb.shape == (M, 128)
+    x = out.to(torch.float64).clone()
+    third = N // 3
+    sin, cos = rotemb[:, 0::2].to(torch.float64), rotemb[:, 1::2].to(torch.float64)  # [M, 64]
+    for part, w in ((0, norm_q), (1, norm_k)):
+        h = x[:, part * third:(part + 1) * third].reshape(M, third // 128, 128)
+        coef = torch.rsqrt((h * h).mean(dim=-1, keepdim=True) + eps)
+        h = h * coef * w.to(torch.float64)[None, None, :]
+        a, b = h[..., 0::2], h[..., 1::2]
+        r = torch.stack((a * cos[:, None, :] - b * sin[:, None, :], a * sin[:, None, :] + b * cos[:, None, :]), dim=-1)
+        x[:, part * third:(part + 1) * third] = r.reshape(M, third)
+    return x.to(torch.float32)

@@ -30,9 +30,10 @@ def test_header_symbols_are_exported(lib):
 
 
 def test_struct_sizes_match_header_layout():
-    # 6 pointers + 4 int64 + 2 int32 ; 16 pointers + 7 int64 + float + 3 int32
+    # 6 pointers + 4 int64 + 2 int32 ; 16 pointers + 7 int64 + float + 3 int32, then 3 pointers + int64 +
+    # float (padded to 8)
     assert ctypes.sizeof(nv.QuantizeArgs) == 6 * 8 + 4 * 8 + 2 * 4
-    assert ctypes.sizeof(nv.GemmArgs) == 16 * 8 + 7 * 8 + 4 * 4
+    assert ctypes.sizeof(nv.GemmArgs) == 16 * 8 + 7 * 8 + 4 * 4 + 3 * 8 + 8 + 8
 
 
 def test_quantize_rejects_bad_arguments(lib):
@@ -87,6 +88,19 @@ def test_gemm_rejects_bad_arguments(lib):
     bad = nv.GemmArgs.from_buffer_copy(a)
     bad.wcscales = 16
     assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
+    # the norm + rotary epilogue: needs both norm weights, three equal parts of whole heads, enough table rows
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.norm_q = 16
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    bad.norm_k = 16
+    bad.rotary_emb = 16
+    bad.rot_rows = 256
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    assert b"three equal parts" in lib.svdq_last_error()
+    bad.N = bad.N_out = 384
+    bad.rot_rows = 128
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    assert b"rows" in lib.svdq_last_error()
 
 
 def test_repack_rejects_bad_arguments(lib):
@@ -98,6 +112,8 @@ def test_repack_rejects_bad_arguments(lib):
     assert lib.svdq_repack_smooth(16, 32, 64, None) == -1
     assert lib.svdq_repack_lora_down(16, 32, 128, 8, None) == -1
     assert lib.svdq_repack_lora_up(16, 32, 8, 16, None) == -1
+    assert lib.svdq_repack_rotemb(16, 32, 48, None) == -1  # rows not a multiple of 32
+    assert lib.svdq_repack_rotemb(16, 16, 64, None) == -1  # in place
 
 
 def test_python_wrappers_refuse_cpu_tensors():
@@ -109,7 +125,7 @@ def test_python_wrappers_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU"):
         svdq_quantize_w4a4_act_fuse_lora(x, lora_down=torch.zeros(128, 16, dtype=torch.bfloat16))
     with pytest.raises(NotImplementedError):
-        svdq_gemm_w4a4(act=x, wgt=x, rotary_emb=x)
+        svdq_gemm_w4a4(act=x, wgt=x, out_q=x)
     with pytest.raises(RuntimeError, match="GPU"):
         svdq_gemm_w4a4(act=x.view(torch.uint8), wgt=x.view(torch.int8), ascales=x, wscales=x, out=x)
 

@@ -135,4 +135,4 @@ def test_gemm_unsupported_raises(dev):
 
     z = torch.zeros(256, 64, dtype=torch.uint8, device=dev)
     with pytest.raises(NotImplementedError):
-        svdq_gemm_w4a4(act=z, wgt=z.view(torch.int8), ascales=z, wscales=z, out=z, norm_q=z)
+        svdq_gemm_w4a4(act=z, wgt=z.view(torch.int8), ascales=z, wscales=z, out=z, poolout=z)

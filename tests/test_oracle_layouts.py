@@ -84,3 +84,29 @@ def test_qweight_first_words_by_hand():
     codes[8, :8] = 3
     w = L.pack_qweight(codes).reshape(-1).view(np.uint32)
     assert w[0] == 0x76543210 and w[1] == 0x77777777 and w[2] == 0x33333333 and w[3] == 0
+
+
+def test_rotemb_two_derivations_agree():
+    """The permute recipe of pack_rotemb (embeddings.py:88-120) against the closed form read off the
+    kernel's loader (epilogues.cuh:282-305,383-401), and pack / unpack as inverses."""
+    rng = np.random.default_rng(0)
+    for M, D in ((16, 8), (32, 128), (48, 64)):
+        logical = rng.standard_normal((M, D)).astype(np.float32)
+        packed = L.pack_rotemb(logical)
+        row, col = L.rotemb_index(M, D)
+        assert np.array_equal(packed.reshape(-1), logical[row, col])
+        assert np.array_equal(L.unpack_rotemb(packed), logical)
+
+
+def test_rotemb_known_positions():
+    """Hand-evaluated positions of the m16n8 fp32 accumulator fragment (the table named in
+    embeddings.py:109-113): thread 4g+t holds c0,c1 = row g, columns 2t, 2t+1 and c2,c3 = row g+8."""
+    M, D = 16, 8
+    logical = (np.arange(M)[:, None] * 100 + np.arange(D)[None, :]).astype(np.float32)
+    packed = L.pack_rotemb(logical).reshape(-1)
+    # lane 0: rows 0 and 8, columns 0, 1
+    assert packed[0:4].tolist() == [0.0, 1.0, 800.0, 801.0]
+    # lane 5 = (g 1, t 1): rows 1 and 9, columns 2, 3
+    assert packed[20:24].tolist() == [102.0, 103.0, 902.0, 903.0]
+    # lane 31 = (g 7, t 3): rows 7 and 15, columns 6, 7
+    assert packed[124:128].tolist() == [706.0, 707.0, 1506.0, 1507.0]
