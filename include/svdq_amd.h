@@ -117,7 +117,8 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * launch_impl.cuh:107, and only NVFP4 layers carry wcscales): SVDQ_EUNSUPPORTED otherwise.
  *
  * Workspace: the work is split evenly over one workgroup per compute unit, so an output tile can be
- * shared by two workgroups, which exchange fp32 partial sums through device memory.  Unless the
+ * shared by two workgroups (by more when there are fewer tiles than compute units: the tiles are then
+ * split along K), which exchange fp32 partial sums through device memory.  Unless the
  * number of 256x256 output tiles is a multiple of the number of compute units (or smaller), the
  * call needs a workspace of 512 KB per compute unit (128 MB on MI355X) plus 4 bytes per tile.  The
  * library allocates it with hipMalloc the first time a (device, stream) pair needs it (that call is
