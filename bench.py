@@ -29,6 +29,9 @@ WORKLOADS = {
     "flux_mlp_fc2": dict(M=4608, K=12288, N=3072, R=32, seed=2),
     "qwen_batched_r128": dict(M=18432, K=3072, N=12288, R=128, seed=4),
     "c1_small": dict(M=256, K=3072, N=3072, R=32, seed=0),
+    # NVFP4 variant of the FLUX single-block layers: fused QKV + MLP-in projection, and the output projection
+    "flux_single_nvfp4": dict(M=4608, K=3072, N=21504, R=32, seed=3, fp4=True),
+    "flux_single_out_nvfp4": dict(M=4608, K=15360, N=3072, R=32, seed=3, fp4=True),
 }
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, the peak the metric is quoted against
 # HBM-side bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
@@ -46,7 +49,9 @@ def cpu_baseline(layer, x, rows: int, iters: int = 20):
 
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    ref = olin.FakeQuantLinear(layer.wq, layer.ws, layer.smooth, layer.proj_down, layer.proj_up, layer.bias)
+    ref = olin.FakeQuantLinear(layer.wq, layer.ws, layer.smooth, layer.proj_down, layer.proj_up, layer.bias,
+                               fp4=layer.fp4, wtscale=float(torch.tensor(layer.wtscale).to(torch.bfloat16)) if layer.fp4 else 1.0,
+                               wcscales=layer.wcscales)
     xs = x[:rows].contiguous()
     times = []
     for _ in range(iters):
@@ -123,16 +128,17 @@ def main():
     cfg = WORKLOADS[args.workload]
     M, K, N, R = cfg["M"], cfg["K"], cfg["N"], cfg["R"]
     dev = torch.device("cuda:0")
-    layer = synth.make_layer(N, K, R, seed=cfg["seed"])
+    fp4 = bool(cfg.get("fp4"))
+    layer = synth.make_layer(N, K, R, seed=cfg["seed"], fp4=fp4)
     x = synth.make_activations(M, K, seed=cfg["seed"])
-    mod = SVDQW4A4Linear(K, N, rank=R, device=dev)
+    mod = SVDQW4A4Linear(K, N, rank=R, precision="nvfp4" if fp4 else "int4", device=dev)
     mod.load_state_dict(synth.to_reference_checkpoint(layer))
     mod.native_tensors()  # load-time repack happens once, outside the timed region
     xd = x.to(dev)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     M_pad = (M + 255) // 256 * 256
     qx = torch.empty(M_pad, K // 2, dtype=torch.uint8, device=dev)
-    asc = torch.empty(K // 64, M_pad, dtype=torch.bfloat16, device=dev)
+    asc = torch.empty(K // 16, M_pad, dtype=torch.float8_e4m3fn, device=dev) if fp4 else torch.empty(K // 64, M_pad, dtype=torch.bfloat16, device=dev)
     la = torch.empty(M_pad, R, dtype=torch.float32, device=dev)
     t = mod.native_tensors()
     from nunchaku_amd.ops import svdq_quantize_w4a4_act_fuse_lora
@@ -158,18 +164,18 @@ def main():
                            lora_up=t["proj_up"], bias=t["bias"], norm_q=nq, norm_k=nk, rotary_emb=rot)
 
     def step():
-        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"], fp4=fp4)
         gemm()
 
     if args.only:
-        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"], fp4=fp4)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
             if args.only == "gemm":
                 gemm()
             else:
-                svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+                svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"], fp4=fp4)
         torch.cuda.synchronize()
         print(f"{args.only}: {(time.perf_counter() - t0) * 1e6 / args.steps:.1f} us per launch (host clock, {args.steps} launches)")
         return
@@ -188,7 +194,7 @@ def main():
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
     for e in evs:
         e[0].record()
-        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"])
+        svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"], fp4=fp4)
         e[1].record()
         gemm()
         e[2].record()
@@ -198,7 +204,7 @@ def main():
 
     ops_layer = 2.0 * M * N * K + 2.0 * M * R * (K + N)
     ops_gemm = 2.0 * M * N * K + 2.0 * M * R * N
-    bytes_quant = 2.0 * M * K + M * K / 2 + 2.0 * M * K / 64 + 4.0 * M * R + 2.0 * K * R + 2.0 * K
+    bytes_quant = 2.0 * M * K + M * K / 2 + (M * K / 16 if fp4 else 2.0 * M * K / 64) + 4.0 * M * R + 2.0 * K * R + 2.0 * K
     value = ops_layer / (ms_per_step * 1e-3) / 1e12
     gemm_tops = ops_gemm / (tg_us * 1e-6) / 1e12
     res = {
@@ -206,7 +212,7 @@ def main():
         "value": value, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: SVDQW4A4Linear forward M={M} K={K} N={N} rank={R} INT4 g64 bf16 in/out"
+        "config": {"workload": f"{args.workload}: SVDQW4A4Linear forward M={M} K={K} N={N} rank={R} {'NVFP4 g16' if fp4 else 'INT4 g64'} bf16 in/out"
                                + (" + RMS norm and rotary embedding on q, k in the GEMM epilogue" if args.qkv_rope else ""),
                    "M": M, "K": K, "N": N, "rank": R},
         "pct_of_int8_mfma_peak": 100.0 * value / INT8_PEAK_TOPS,
@@ -218,7 +224,7 @@ def main():
             "gemm_main_term_TOPS": 2.0 * M * N * K / (tg_us * 1e-6) / 1e12,
         },
         "roofline": {
-            "kernel": "gemm_w4a4_kernel<false, false, true>" if args.qkv_rope else "gemm_w4a4_kernel<false, false, false>", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
+            "kernel": f"gemm_w4a4_kernel<false, {'true' if fp4 else 'false'}, {'true' if args.qkv_rope else 'false'}>", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
             "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": PROFILED_GEMM_TRAFFIC_BYTES.get(args.workload),
             "peak_basis": "dense INT8 MFMA (the metric's peak); the kernel issues fp16 MFMA, dense peak 2500",
             "frac_of_fp16_mfma_peak": gemm_tops / FP16_PEAK_TFLOPS,

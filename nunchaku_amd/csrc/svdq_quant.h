@@ -49,11 +49,12 @@ __device__ inline uint32_t f32_to_e4m3(float s) {
     return (uint32_t)(ex << 3) | ((b >> 20) & 7u);
 }
 
-// fp32 -> 4-bit e2m1 pattern, round to nearest even, saturating at 6
-__device__ inline uint32_t f32_to_e2m1(float v) {
-    const float a = fabsf(v);
+// fp32 -> 4-bit e2m1 pattern, round to nearest even, saturating at 6: the rule the hardware conversion
+// below implements (grid 0 .5 1 1.5 2 3 4 6; ties go to the pattern with an even low bit; the sign bit
+// is kept, also for zero).  Kept as the statement of the rule and for host-side checks.
+__host__ __device__ inline uint32_t f32_to_e2m1(float v) {
+    const float a = v < 0.f ? -v : v;
     uint32_t c;
-    // grid 0 .5 1 1.5 2 3 4 6 ; ties go to the pattern with an even low bit
     if (a <= 0.25f) c = 0;
     else if (a < 0.75f) c = 1;
     else if (a <= 1.25f) c = 2;
@@ -63,6 +64,18 @@ __device__ inline uint32_t f32_to_e2m1(float v) {
     else if (a <= 5.0f) c = 6;
     else c = 7;
     return c | ((f32_bits(v) >> 28) & 8u);
+}
+
+// 8 fp32 -> one word of e2m1 patterns (element j in bits [4j, 4j+4)) with the hardware conversion
+// v_cvt_scalef32_pk_fp4_f32 at scale 1: two values per instruction.  It agrees with f32_to_e2m1 on
+// every non-NaN fp32 bit pattern (checked exhaustively on gfx950).
+__device__ inline uint32_t pack8_e2m1(const float (&t)[8]) {
+    uint32_t w = 0;
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[0], t[1], 1.0f, 0);
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[2], t[3], 1.0f, 1);
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[4], t[5], 1.0f, 2);
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[6], t[7], 1.0f, 3);
+    return w;
 }
 
 
@@ -106,10 +119,11 @@ __device__ inline void quantize_nvfp4_two_groups(const float (&y)[32], u32x4_t &
         sc[h] = f32_to_e4m3(s);
 #pragma unroll
         for (int wi = 0; wi < 2; wi++) {
-            uint32_t w = 0;
+            float t[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) w |= f32_to_e2m1(s > 0.f ? __fmul_rn(y[16 * h + 8 * wi + j], rcp) : 0.f) << (4 * j);
-            words[2 * h + wi] = w;
+            for (int j = 0; j < 8; j++) t[j] = __fmul_rn(y[16 * h + 8 * wi + j], rcp);
+            // (a zero group gives codes 0 whatever the signs of its zeros)
+            words[2 * h + wi] = s > 0.f ? pack8_e2m1(t) : 0u;
         }
     }
 }
