@@ -126,7 +126,8 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * for every later call on that pair; at most 16 pairs.  Calls on one stream run in order and share
  * the workspace safely; the same stream must not be used from two threads at once.  Setting the
  * environment variable SVDQ_GEMM_NO_SHARED_TILES makes every call use whole tiles only (no workspace,
- * slower when the tile count does not divide evenly).
+ * slower when the tile count does not divide evenly).  With fewer tiles than compute units a workgroup gets at least
+ * 12 units (of 128 along K) of work; SVDQ_GEMM_MIN_UNITS overrides that number.
  * ------------------------------------------------------------------------------------------ */
 typedef struct svdq_gemm_args {
     const void *act;        /* u8 native activation tiles [M_pad, K/2]                              */

@@ -172,10 +172,15 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     if (getenv("SVDQ_GEMM_NO_SHARED_TILES")) {  // whole tiles only: the largest workgroup count that divides the tile count
         while (ntiles % nwg != 0) nwg--;
     } else if (ntiles < ncu) {
-        // fewer tiles than compute units: several workgroups per tile, each with at least four units (eight
-        // k-groups) of work, so that the fixed cost of a workgroup and of adding up the parts stays small
+        // fewer tiles than compute units: several workgroups per tile, each with at least 12 units (24
+        // k-groups) of work.  The fixed cost of a workgroup and of adding up the parked parts (one round
+        // trip to memory per part and 32-row slab) outweighs a finer split: M=256, K=N=3072 takes 119 us
+        // with 4 units per workgroup, 79 with 8, 71 with 12, 75 unsplit.  SVDQ_GEMM_MIN_UNITS overrides
+        // the number (the tests use it to reach splits among many workgroups).
         const long long units = (long long)ntiles * (a->K / 128);
-        long long w = units / 4;
+        const char *mu = getenv("SVDQ_GEMM_MIN_UNITS");
+        const int min_units = mu && atoi(mu) > 0 ? atoi(mu) : 12;
+        long long w = units / min_units;
         if (w > ncu) w = ncu;
         if (w > nwg) nwg = (int)w;
     }

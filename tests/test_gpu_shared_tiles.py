@@ -38,12 +38,13 @@ def test_shared_tiles_match_whole_tiles(dev, M, K, N, R):
 
 
 @pytest.mark.parametrize("M,K,N,R", [(256, 3072, 3072, 32), (256, 1024, 512, 16), (512, 12288, 256, 32), (300, 640, 768, 32)])
-def test_few_tiles_split_among_many_workgroups(dev, M, K, N, R):
+def test_few_tiles_split_among_many_workgroups(dev, M, K, N, R, monkeypatch):
     """Fewer tiles than compute units: every tile is split along K among several workgroups (6, 2, 24
     parties; K = 640 gives shares that straddle tile boundaries), the last to arrive adds up the rest."""
     M_pad = (M + 255) // 256 * 256
     ntiles = (M_pad // 256) * ((N + 255) // 256)
     ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    monkeypatch.setenv("SVDQ_GEMM_MIN_UNITS", "4")  # (the default of 12 units per workgroup would split only the third shape)
     assert ntiles < ncu and ntiles * (K // 128) // 4 > ntiles, "the shape must give several workgroups per tile"
     # (more parties, more fp32 additions in another order: more elements whose bf16 rounding flips)
     _compare_with_whole_tiles(dev, M, K, N, R, max_fraction_different=2e-2)
