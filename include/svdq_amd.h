@@ -172,6 +172,27 @@ typedef struct svdq_gemm_args {
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
 
+/* ------------------------------------------------------------------------------------------
+ * AWQ W4A16 GEMV (the other quantized linear of the reference's models: modulation layers, text
+ * encoder), for 1..8 rows of x.  Replaces ops.gemv_awq (nunchaku/ops/gemv.py ->
+ * src/kernels/awq/gemv_awq.cu:84-294) and the bias add of AWQW4A16Linear.forward
+ * (nunchaku/models/linear.py:172-186).  out[m, n] = sum_k bf16(code[n, k] * scales[k/64, n] +
+ * zeros[k/64, n]) * x[m, k], fp32 accumulation, bf16 result (+ bias, added to the bf16 result).
+ * qweight is read in the reference's own storage (no repack).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct svdq_awq_gemv_args {
+    const void *x;        /* bf16 [M, K] row-major                                                   */
+    const void *qweight;  /* int32 [N/4, K/2] as stored by the reference (tinychat_utils.py:76-106)  */
+    const void *scales;   /* bf16 [K/64, N]                                                          */
+    const void *zeros;    /* bf16 [K/64, N]: minus the scaled zero point                             */
+    const void *bias;     /* bf16 [N] or NULL                                                        */
+    void *out;            /* bf16 [M, N] row-major                                                   */
+    int64_t M, N, K;      /* 1 <= M <= 8 (gemv_awq.cu:262), N % 4 == 0, K % 64 == 0                  */
+    int32_t group_size;   /* must be 64 (gemv_awq.cu:263)                                            */
+} svdq_awq_gemv_args;
+
+int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream);
+
 
 
 

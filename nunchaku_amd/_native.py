@@ -19,7 +19,7 @@ _PKG_DIR = Path(__file__).resolve().parent
 _CSRC = _PKG_DIR / "csrc"
 LIB_PATH = _PKG_DIR / "libsvdq_amd.so"
 PROBE_LIB_PATH = _PKG_DIR / "libsvdq_probe.so"  # bench.py's MFMA-rate probe (csrc/probe_mfma_rate.hip)
-SOURCES = ["repack.hip", "quantize.hip", "gemm.hip"]
+SOURCES = ["repack.hip", "quantize.hip", "gemm.hip", "awq_gemv.hip"]
 HIPCC_FLAGS = [
     "-shared", "-fPIC", "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -30,7 +30,7 @@ EXPORTED_SYMBOLS = [
     "svdq_abi_version", "svdq_last_error",
     "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
     "svdq_repack_smooth", "svdq_repack_lora_down", "svdq_repack_lora_up", "svdq_repack_rotemb",
-    "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4",
+    "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4", "svdq_awq_gemv_w4a16",
 ]
 
 
@@ -62,6 +62,16 @@ class GemmArgs(ctypes.Structure):
         ("fp4", ctypes.c_int32),
         ("norm_q", ctypes.c_void_p), ("norm_k", ctypes.c_void_p), ("rotary_emb", ctypes.c_void_p),
         ("rot_rows", ctypes.c_int64), ("norm_eps", ctypes.c_float),
+    ]
+
+
+class AwqGemvArgs(ctypes.Structure):
+    """Mirror of ``svdq_awq_gemv_args``."""
+
+    _fields_ = [
+        ("x", ctypes.c_void_p), ("qweight", ctypes.c_void_p), ("scales", ctypes.c_void_p), ("zeros", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p), ("out", ctypes.c_void_p),
+        ("M", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64), ("group_size", ctypes.c_int32),
     ]
 
 
@@ -130,6 +140,7 @@ def lib() -> ctypes.CDLL:
         L.svdq_repack_rotemb.argtypes = [vp, vp, i64, vp]
         L.svdq_quantize_w4a4_act_fuse_lora.argtypes = [ctypes.POINTER(QuantizeArgs), vp]
         L.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), vp]
         for name in EXPORTED_SYMBOLS:
             getattr(L, name)
             if name not in ("svdq_last_error",):

@@ -1,3 +1,3 @@
-from .linear import SVDQW4A4Linear
+from .linear import AWQW4A16Linear, SVDQW4A4Linear
 
-__all__ = ["SVDQW4A4Linear"]
+__all__ = ["SVDQW4A4Linear", "AWQW4A16Linear"]

@@ -152,3 +152,38 @@ class SVDQW4A4Linear(nn.Module):
             f"SVDQW4A4Linear(in_features={self.in_features}, out_features={self.out_features}, rank={self.rank}, "
             f"precision={self.precision}, act_unsigned={self.act_unsigned})"
         )
+
+
+class AWQW4A16Linear(nn.Module):
+    """AWQ W4A16 linear for a handful of rows (modulation layers, text encoder), parameters as in
+    nunchaku/models/linear.py:138-208: qweight int32 [N/4, K/2], wscales / wzeros bf16 [K/G, N], bias
+    bf16 [N]; the tensors are used in the reference's storage as they are."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, group_size: int = 64,
+                 torch_dtype: torch.dtype = torch.bfloat16, device: str | torch.device | None = None):
+        super().__init__()
+        if device is None:
+            device = torch.device("cpu")
+        self.in_features, self.out_features, self.group_size = in_features, out_features, group_size
+        self.qweight = nn.Parameter(torch.empty(out_features // 4, in_features // 2, dtype=torch.int32, device=device), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(out_features, dtype=torch_dtype, device=device), requires_grad=True) if bias else None
+        self.wscales = nn.Parameter(torch.empty(in_features // group_size, out_features, dtype=torch_dtype, device=device), requires_grad=False)
+        self.wzeros = nn.Parameter(torch.empty(in_features // group_size, out_features, dtype=torch_dtype, device=device), requires_grad=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from ..ops.gemv import awq_gemv_w4a16
+
+        x = x.contiguous()
+        return awq_gemv_w4a16(
+            in_feats=x, kernel=self.qweight, scaling_factors=self.wscales, zeros=self.wzeros,
+            m=x.numel() // x.shape[-1], n=self.out_features, k=self.in_features, group_size=self.group_size,
+            bias=None if self.bias is None else self.bias.detach(),
+        )
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, group_size: int = 64, torch_dtype: torch.dtype = torch.bfloat16, device: str = "cpu", **kwargs):
+        return cls(linear.in_features, linear.out_features, bias=linear.bias is not None, group_size=group_size,
+                   torch_dtype=torch_dtype, device=device)
+
+    def __repr__(self):
+        return f"AWQW4A16Linear(in_features={self.in_features}, out_features={self.out_features}, group_size={self.group_size})"

@@ -103,6 +103,15 @@ def test_gemm_rejects_bad_arguments(lib):
     assert b"rows" in lib.svdq_last_error()
 
 
+def test_awq_gemv_rejects_bad_arguments(lib):
+    assert lib.svdq_awq_gemv_w4a16(None, None) == -1
+    a = nv.AwqGemvArgs(x=16, qweight=16, scales=16, zeros=16, out=16, M=1, N=64, K=128, group_size=64)
+    for field, value, code in (("M", 9, -1), ("M", 0, -1), ("N", 6, -1), ("K", 100, -1), ("group_size", 128, -2), ("x", 8, -1), ("out", None, -1)):
+        bad = nv.AwqGemvArgs.from_buffer_copy(a)
+        setattr(bad, field, value)
+        assert lib.svdq_awq_gemv_w4a16(ctypes.byref(bad), None) == code, field
+
+
 def test_repack_rejects_bad_arguments(lib):
     assert lib.svdq_repack_qweight(None, None, 128, 128, 0, None) == -1
     assert lib.svdq_repack_qweight(16, 32, 100, 128, 0, None) == -1
