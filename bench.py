@@ -98,10 +98,11 @@ def main():
     ap.add_argument("--qkv-rope", action="store_true",
                     help="time the GEMM with the RMS-norm + rotary epilogue of fused_qkv_norm_rottary (workload flux_qkv); "
                          "the CPU comparison is skipped")
-    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "mfma-rate"], default=None,
+    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "mfma-rate", "awq-gemv"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
                          "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters; "
-                         "'mfma-rate' measures the MFMA instruction of the GEMM alone")
+                         "'mfma-rate' measures the MFMA instruction of the GEMM alone; "
+                         "'awq-gemv' times the AWQ W4A16 GEMV at the modulation shape (1 row, K=3072, N=18432)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -112,6 +113,30 @@ def main():
     if args.only == "mfma-rate":
         torch.cuda.init()
         print(f"mfma-rate: v_mfma_f32_32x32x16_f16 alone, TFLOP/s: {mfma_rate_probe()}")
+        return
+    if args.only == "awq-gemv":
+        from nunchaku_amd.ops import awq_gemv_w4a16
+
+        K, N = 3072, 18432
+        dev = torch.device("cuda:0")
+        gen = torch.Generator().manual_seed(0)
+        qw = torch.randint(-2**31, 2**31 - 1, (N // 4, K // 2), generator=gen, dtype=torch.int32).to(dev)
+        sc = (0.001 + 0.002 * torch.rand(K // 64, N, generator=gen)).to(torch.bfloat16).to(dev)
+        zr = (-0.02 * torch.rand(K // 64, N, generator=gen)).to(torch.bfloat16).to(dev)
+        bias = (0.02 * torch.randn(N, generator=gen)).to(torch.bfloat16).to(dev)
+        for rows in (1, 4, 8):
+            x = torch.randn(rows, K, generator=gen).to(torch.bfloat16).to(dev)
+            for _ in range(20):
+                awq_gemv_w4a16(x, qw, sc, zr, rows, N, K, bias=bias)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.steps):
+                awq_gemv_w4a16(x, qw, sc, zr, rows, N, K, bias=bias)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / args.steps
+            nbytes = N * K / 2 + 2 * 2 * (K // 64) * N + 2 * N + rows * (K + N) * 2  # codes, scales + zeros, bias, x and out
+            print(f"awq-gemv rows={rows} K={K} N={N}: {us:.2f} us per launch (back to back), {nbytes / us / 1e3:.0f} GB/s of {nbytes / 1e6:.1f} MB")
         return
     if args.only == "copy":
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(1)

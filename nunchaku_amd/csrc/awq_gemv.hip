@@ -28,11 +28,24 @@ struct AwqParams {
 
 typedef __bf16 bf16x2_v __attribute__((ext_vector_type(2)));
 
-template <int MT>
+// XLDS: the rows of x are copied to LDS once per workgroup (every wave needs all of x; from global memory
+// the activation loads, 64 bytes per lane, row of x and step, outweigh the weight stream from 2 rows on).
+template <int MT, bool XLDS>
 __global__ void __launch_bounds__(256) awq_gemv_kernel(AwqParams p) {
+    extern __shared__ u32x4_t xlds[];  // [M][K] bf16
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int rg = blockIdx.x * 4 + wave;  // 4-row group
+    if (XLDS) {
+        const int n16 = p.M * p.K / 8;
+        for (int i = threadIdx.x; i < n16; i += 256) xlds[i] = ((const u32x4_t *)p.x)[i];
+        __syncthreads();
+    }
+    // Workgroups are dealt to the 8 XCDs in turn (blockIdx % 8), each with its own L2.  A 128-byte line of
+    // scales or zeros serves 64 output rows = 16 row groups = 4 workgroups: consecutive workgroups of the
+    // row order are therefore given to the same XCD, so that the line is fetched from memory once, not 8 times.
+    int wg = blockIdx.x;
+    if (gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+    const int rg = wg * 4 + wave;  // 4-row group
     if (rg * 4 >= p.N) return;
     const int u = lane & 7, blk = lane >> 3;
     const int row = rg * 4 + (u >> 1);
@@ -44,21 +57,25 @@ __global__ void __launch_bounds__(256) awq_gemv_kernel(AwqParams p) {
 #pragma unroll
     for (int m = 0; m < MT; m++) acc[m] = 0.f;
 
-    auto load_w = [&](int it, u32x4_t &w, float &s, float &z) {
-        const int kb = it * 8 + blk;
-        const bool ok = kb < kblocks;
-        w = ok ? __builtin_nontemporal_load(wp + it * 64) : u32x4_t{0, 0, 0, 0};
-        // (a block past the end contributes nothing: scale and zero 0)
-        s = ok ? bf16_bits_to_f32(p.scales[(size_t)kb * p.N + row]) : 0.f;
-        z = ok ? bf16_bits_to_f32(p.zeros[(size_t)kb * p.N + row]) : 0.f;
+    // Weights, scales and zeros are requested DEPTH steps ahead (a ring of DEPTH + 1 register sets, indexed
+    // statically).  Every request is unconditional: a step or channel block past the end re-reads the last
+    // valid one and gets scale and zero 0, so that it contributes nothing; a request behind a branch would make
+    // the compiler's wait counting assume the worst and wait for the requests made ahead.
+    constexpr int DEPTH = 3;
+    u32x4_t wq[DEPTH + 1];
+    uint16_t sq[DEPTH + 1], zq[DEPTH + 1];
+    auto load_w = [&](int it, int slot) {
+        int kb = it * 8 + blk;
+        kb = kb < kblocks ? kb : kblocks - 1;
+        wq[slot] = __builtin_nontemporal_load((const u32x4_t *)(p.qweight + ((size_t)rg * kblocks + kb) * 128) + u);
+        sq[slot] = p.scales[(size_t)kb * p.N + row];
+        zq[slot] = p.zeros[(size_t)kb * p.N + row];
     };
-    u32x4_t w_next;
-    float s_next, z_next;
-    load_w(0, w_next, s_next, z_next);
-    for (int it = 0; it < iters; it++) {
-        const u32x4_t w = w_next;
-        const float s = s_next, z = z_next;
-        if (it + 1 < iters) load_w(it + 1, w_next, s_next, z_next);
+    auto step = [&](int it, int slot) {
+        const bool ok = it * 8 + blk < kblocks;
+        const u32x4_t w = wq[slot];
+        const float s = ok ? bf16_bits_to_f32(sq[slot]) : 0.f, z = ok ? bf16_bits_to_f32(zq[slot]) : 0.f;
+        load_w(it + DEPTH, slot == 0 ? DEPTH : slot - 1);  // the set freed by the previous step ... see the ring below
         // activations of this lane's 32 channels for every row of x (a channel block past the end is
         // clamped to the last one: its weights are zero)
         int kb = it * 8 + blk;
@@ -67,7 +84,8 @@ __global__ void __launch_bounds__(256) awq_gemv_kernel(AwqParams p) {
         uint32_t xv[MT][16];
 #pragma unroll
         for (int m = 0; m < MT; m++) {
-            const u32x4_t *xp = (const u32x4_t *)(p.x + (size_t)(m < p.M ? m : p.M - 1) * p.K + k0);
+            const size_t xoff = (size_t)(m < p.M ? m : p.M - 1) * p.K + k0;
+            const u32x4_t *xp = XLDS ? xlds + xoff / 8 : (const u32x4_t *)(p.x + xoff);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const u32x4_t v = xp[i];
@@ -89,11 +107,21 @@ __global__ void __launch_bounds__(256) awq_gemv_kernel(AwqParams p) {
                 const int xw = i2 + 4 * pq;  // channels 8 pq + 2 i2 + {0, 1} = word 4 pq + i2 of the lane's 16
 #pragma unroll
                 for (int m = 0; m < MT; m++)
-                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, pair), __builtin_bit_cast(bf16x2_v, xv[m][xw]),
-                                                             acc[m], false);
+                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, pair), __builtin_bit_cast(bf16x2_v, xv[m][xw]), acc[m], false);
             }
         }
+    };
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) load_w(d, d);
+    // step it uses set it % (DEPTH + 1) and refills the set of step it - 1, which is (it + DEPTH) % (DEPTH + 1)
+    for (int it0 = 0; it0 < iters; it0 += DEPTH + 1) {
+#pragma unroll
+        for (int sl = 0; sl <= DEPTH; sl++) {
+            if (it0 + sl >= iters) goto done;
+            step(it0 + sl, sl);
+        }
     }
+done:
     // lanes with the same (l % 8) / 2 hold parts of the same row
 #pragma unroll
     for (int m = 0; m < MT; m++) {
@@ -113,7 +141,18 @@ __global__ void __launch_bounds__(256) awq_gemv_kernel(AwqParams p) {
 
 template <int MT>
 int launch(const AwqParams &p, hipStream_t stream) {
-    hipLaunchKernelGGL(awq_gemv_kernel<MT>, dim3((p.N / 4 + 3) / 4), dim3(256), 0, stream, p);
+    const size_t xbytes = (size_t)p.M * p.K * 2;
+    const dim3 grid((p.N / 4 + 3) / 4);
+    if (xbytes <= 64 * 1024) {
+        auto kern = awq_gemv_kernel<MT, true>;
+        if (xbytes > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)xbytes);
+            if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "awq_gemv: cannot reserve %zu bytes of LDS: %s", xbytes, hipGetErrorString(e));
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(256), xbytes, stream, p);
+    } else {
+        hipLaunchKernelGGL((awq_gemv_kernel<MT, false>), grid, dim3(256), 0, stream, p);
+    }
     return check_launch("awq_gemv_w4a16");
 }
 

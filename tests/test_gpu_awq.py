@@ -48,6 +48,18 @@ def test_against_oracle(dev, rows, oc, ic):
     _check(y, awq.gemv(x, codes, scales, zeros), bias)
 
 
+def test_long_k_takes_the_path_without_lds_staging(dev):
+    """8 rows of K=4160 do not fit the 64 KB the kernel stages x in: the activations then come from global memory."""
+    oc, ic, rows = 64, 4160, 8
+    announce(f"awq gemv rows={rows} oc={oc} ic={ic} (x not staged)")
+    m, (codes, scales, zeros, bias) = _module(dev, oc, ic, seed=77)
+    x = torch.randn(rows, ic, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    y = m(x.to(dev))
+    torch.cuda.synchronize()
+    _check(y, awq.gemv(x, codes, scales, zeros), bias)
+    _check(m(x[:1].to(dev)), awq.gemv(x[:1], codes, scales, zeros), bias)  # one row of the same layer: staged
+
+
 def test_modulation_shape_and_linearity(dev):
     """K=3072, N=18432 (six modulation vectors of a 3072-wide block), one row; without bias the result is
     linear in x up to the bf16 rounding of the output."""
