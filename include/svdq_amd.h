@@ -136,7 +136,8 @@ typedef struct svdq_gemm_args {
     const void *wscales;    /* native fp16 scales (svdq_repack_wscales / _wmscales)                 */
     const float *colnorm;   /* fp32 [N] from the same repack call                                   */
     const void *bias;       /* bf16 [N] channel order, or NULL                                      */
-    const void *wcscales;   /* bf16 [N] channel order, or NULL                                      */
+    const void *wcscales;   /* bf16 [N] channel order, or NULL; no element may be zero (the low-rank
+                               term is added in units of the column factor)                         */
     const float *lora_act_in; /* fp32 [M_pad, R_up] row-major, or NULL                              */
     const void *lora_up;    /* bf16 [N, R_up] (svdq_repack_lora_up), or NULL                        */
     const float *lora_scales; /* HOST pointer, ceil(R_up/16) floats, or NULL for all ones           */

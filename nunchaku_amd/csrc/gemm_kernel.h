@@ -188,7 +188,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         int m0, n0, shift;
         bool col_ok;
         const uint8_t *a_base[2], *b_base[2], *as_base, *bs_base;
-        uint32_t bs_voff;
     };
     // follow: the segment after the one given by prev_* (the next tile, from its first k-group), without divisions
     auto make_ctx = [&](int sidx, int slot, int tid, bool follow, int prev_tile, int prev_m0, int prev_n0) {
@@ -209,7 +208,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             tile_coords(c.tile, c.m0, c.n0);
         }
         c.shift = rowshift[slot * 256 + tid];  // thread tid stages the scales of row tid
-        c.col_ok = c.n0 + tid < p.N;
+        c.col_ok = c.n0 + ca * 64 < p.N;  // (N is a multiple of 128: a wave's 64 columns are inside or outside together)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int t = ca + 4 * j;
@@ -221,8 +220,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         // scale sources: INT4 one bf16 / fp16 value per (group, row / column); NVFP4 one word of four
         // e4m3 (activations) or four fp16 (weights) per (64-group, row / column)
         c.as_base = (const uint8_t *)p.ascales + (size_t)(c.m0 + ca * 64) * AS_ELT;  // row m0 + tid = m0 + 64 ca + lane
-        c.bs_base = (const uint8_t *)p.wscales + (size_t)c.n0 * BS_ELT;
-        c.bs_voff = (uint32_t)(c.col_ok ? tid : p.N - 1 - c.n0) * BS_ELT;
+        // column n0 + tid = n0 + 64 ca + lane; a wave beyond N reads the last 64 columns instead (its scales are
+        // stored as zero), so that the lane part of the offset is the same everywhere and needs no register
+        c.bs_base = (const uint8_t *)p.wscales + (size_t)(c.col_ok ? c.n0 + ca * 64 : p.N - 64) * BS_ELT;
         return c;
     };
 
@@ -260,7 +260,12 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             asm volatile("v_lshrrev_b32 %0, 3, %1" : "=v"(lane_off) : "v"(code_voff));
         else
             asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(lane_off) : "v"(code_voff));
-        const uint32_t va = (uint32_t)gc * as_stride + lane_off, vb = (uint32_t)gc * bs_stride + c.bs_voff;
+        uint32_t lane_off_b;
+        if (!FP4)
+            asm volatile("v_lshrrev_b32 %0, 3, %1" : "=v"(lane_off_b) : "v"(code_voff));
+        else
+            asm volatile("v_lshrrev_b32 %0, 1, %1" : "=v"(lane_off_b) : "v"(code_voff));
+        const uint32_t va = (uint32_t)gc * as_stride + lane_off, vb = (uint32_t)gc * bs_stride + lane_off_b;
         if (!FP4) {
             uint32_t t;
             asm volatile("global_load_ushort %0, %1, %2" : "=v"(ra) : "v"(va), "s"(c.as_base) : "memory");
@@ -316,11 +321,11 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
         if (!FP4) {
             ra = *(const uint16_t *)(c.as_base + (gc * as_stride + as_voff));
-            rb[0] = *(const uint16_t *)(c.bs_base + (gc * bs_stride + c.bs_voff));
+            rb[0] = *(const uint16_t *)(c.bs_base + (gc * bs_stride + lane * BS_ELT));
             rb[1] = 0;
         } else {
             ra = *(const uint32_t *)(c.as_base + (gc * as_stride + as_voff));
-            rb = *(const u32x2_t *)(c.bs_base + (gc * bs_stride + c.bs_voff));
+            rb = *(const u32x2_t *)(c.bs_base + (gc * bs_stride + lane * BS_ELT));
         }
     };
     auto issue_first_stages = [&](const TileCtx &c) {
@@ -637,34 +642,18 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         }
     }
     // Low-rank up projection (lora.cuh:110-241): out += bf16(lora_act * scale) @ up^T on the matrix cores.
-    // INT4: the projection is added to the accumulators BEFORE they are scaled.  The accumulators are in
-    // normalised units (out = acc * rn[row] * cf[col] + bias with rn and cf powers of two: alpha is 1 and
-    // there are no per-channel scales), so the operands are divided by rn and cf first; that only changes
-    // their exponents, the bf16 products are the same numbers.  The matrix cores then update the
-    // accumulators in place and the operands are dead before the output pass starts.
-    // NVFP4: cf is not a power of two; the projection is added after the scaling, inside the output pass.
-    constexpr bool LORA_FIRST = !FP4;
+    // The projection is added to the accumulators BEFORE they are scaled.  The accumulators are in
+    // normalised units (out = acc * rn[row] * cf[col] + bias), so the operands are divided by rn and cf
+    // first; the matrix cores then update the accumulators in place and the operands are dead before the
+    // output pass starts.  INT4: rn and cf are powers of two (alpha is 1 and there are no per-channel
+    // scales), the division only changes exponents and the bf16 products are the same numbers.  NVFP4: cf
+    // (column normalisation x alpha x wcscales) is an arbitrary number, so up / cf is passed as the sum of
+    // two bf16 numbers (the rounded quotient and the rounded remainder: relative error 2^-17, below the
+    // rounding noise of the main loop) in two matrix-core steps; wcscales must not be zero.
     const int nsteps = p.R_up / 16;
-    bf16x8_t la_pre[4][2], lb_pre[4][2];
-    auto load_la = [&](int mt, int s) {
-        const float ls = p.lora_scales[s < 8 ? s : 7];
-        const float4_t *ap = (const float4_t *)(p.lora_act + (size_t)(wrow0 + mt * 32 + r32) * p.R_up + 16 * s + 8 * h);
-        const float4_t v0 = ap[0], v1 = ap[1];
-        u32x4_t w;
-        w[0] = pack_bf16x2(v0[0] * ls, v0[1] * ls);
-        w[1] = pack_bf16x2(v0[2] * ls, v0[3] * ls);
-        w[2] = pack_bf16x2(v1[0] * ls, v1[1] * ls);
-        w[3] = pack_bf16x2(v1[2] * ls, v1[3] * ls);
-        return __builtin_bit_cast(bf16x8_t, w);
-    };
-    auto load_lb = [&](int nt, int s) {
-        const int n = wcol0 + nt * 32 + r32;
-        const u32x4_t bw = n < p.N ? *(const u32x4_t *)(p.lora_up + (size_t)n * p.R_up + 16 * s + 8 * h) : u32x4_t{0, 0, 0, 0};
-        return __builtin_bit_cast(bf16x8_t, bw);
-    };
     SVDQ_STAMP_TILE(ti, 6);
     if (run_epilogue && nsteps > 0) {
-        if (LORA_FIRST) {
+        {
             // two 16-rank steps per round; every request of a round is issued before any of its data is
             // touched, so a round costs one memory latency
             for (int s0 = 0; s0 < nsteps; s0 += 2) {
@@ -683,14 +672,20 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                     const u32x4_t *bp = (const u32x4_t *)(p.lora_up + (size_t)(ok ? n : 0) * p.R_up + 8 * h);
                     rb[t][0] = bp[2 * s0];
                     rb[t][1] = bp[2 * s1];
-                    rcf[t] = ok ? __builtin_amdgcn_rcpf(p.colnorm[n]) : 0.f;  // of a power of two: exact
+                    if (!FP4) {
+                        rcf[t] = ok ? __builtin_amdgcn_rcpf(p.colnorm[n]) : 0.f;  // of a power of two: exact
+                    } else {
+                        float cf = ok ? p.colnorm[n] * p.alpha : 1.f;
+                        if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
+                        rcf[t] = ok ? __fdiv_rn(1.0f, cf) : 0.f;
+                    }
                     lsr[t] = ldexpf(1.0f, tile_shift[wm * 128 + t * 32 + r32]);
                 }
 #pragma unroll
                 for (int k = 0; k < 2; k++) {
                     if (k == 1 && !two) break;
                     const float ls = p.lora_scales[(s0 + k) < 8 ? (s0 + k) : 7];
-                    bf16x8_t la[4], lb[4];
+                    bf16x8_t la[4], lb[4], lb_rem[4];
 #pragma unroll
                     for (int t = 0; t < 4; t++) {
                         const float f = ls * lsr[t];
@@ -701,28 +696,30 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                         w[2] = pack_bf16x2(v1[0] * f, v1[1] * f);
                         w[3] = pack_bf16x2(v1[2] * f, v1[3] * f);
                         la[t] = __builtin_bit_cast(bf16x8_t, w);
-                        u32x4_t bw = rb[t][k];
+                        u32x4_t bw = rb[t][k], br = u32x4_t{0, 0, 0, 0};
 #pragma unroll
-                        for (int i = 0; i < 4; i++)
-                            bw[i] = pack_bf16x2(bits_f32(bw[i] << 16) * rcf[t], bits_f32(bw[i] & 0xFFFF0000u) * rcf[t]);
+                        for (int i = 0; i < 4; i++) {
+                            const float q0 = bits_f32(bw[i] << 16) * rcf[t], q1 = bits_f32(bw[i] & 0xFFFF0000u) * rcf[t];
+                            bw[i] = pack_bf16x2(q0, q1);
+                            if (FP4) br[i] = pack_bf16x2(q0 - bits_f32(bw[i] << 16), q1 - bits_f32(bw[i] & 0xFFFF0000u));
+                        }
                         lb[t] = __builtin_bit_cast(bf16x8_t, bw);
+                        lb_rem[t] = __builtin_bit_cast(bf16x8_t, br);
                     }
 #pragma unroll
                     for (int mt = 0; mt < 4; mt++)
 #pragma unroll
                         for (int nt = 0; nt < 4; nt++)
                             acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb[nt], la[mt], acc[mt][nt], 0, 0, 0);
+                    if (FP4) {
+#pragma unroll
+                        for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+                            for (int nt = 0; nt < 4; nt++)
+                                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb_rem[nt], la[mt], acc[mt][nt], 0, 0, 0);
+                    }
                 }
             }
-        } else {
-#pragma unroll
-            for (int t = 0; t < 4; t++)
-#pragma unroll
-                for (int k = 0; k < 2; k++) {
-                    const int s = k < nsteps ? k : 0;
-                    la_pre[t][k] = load_la(t, s);
-                    lb_pre[t][k] = load_lb(t, s);
-                }
         }
     }
     SVDQ_STAMP_TILE(ti, 7);
@@ -801,21 +798,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-        }
-        if (!LORA_FIRST && nsteps > 0) {
-#pragma unroll
-            for (int k = 0; k < 2; k++)
-                if (k < nsteps) {
-#pragma unroll
-                    for (int nt = 0; nt < 4; nt++)
-                        v[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb_pre[nt][k], la_pre[mt][k], v[nt], 0, 0, 0);
-                }
-            for (int s2 = 2; s2 < nsteps; s2++) {
-                const bf16x8_t la = load_la(mt, s2);
-#pragma unroll
-                for (int nt = 0; nt < 4; nt++)
-                    v[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_lb(nt, s2), la, v[nt], 0, 0, 0);
-            }
         }
         if (NEXT && SVDQ_ROPE_ENABLED && p.rotary && wcol0 < p.rope_cols) {
             // EpilogueRMSNormRope (epilogues.cuh:269-425): the wave's 128 columns are one head of q or k.
