@@ -87,12 +87,13 @@ __device__ inline float e4m3_to_f32(uint32_t b) {
 }
 
 __device__ inline float gelu_tanh(float x) {
-    // x * (0.5 + 0.5 * tanh(0.79788456 * (x + 0.044715 x^3)))   (epilogues.cuh:22-44)
-    const float u = 0.79788456f * (x + 0.044715f * x * x * x);
-    // tanh(u) = 1 - 2 / (exp(2u) + 1); exact enough in fp32 and safe for large |u|
-    const float e = __expf(2.0f * u);
-    const float t = 1.0f - 2.0f / (e + 1.0f);
-    return x * (0.5f + 0.5f * t);
+    // x * (0.5 + 0.5 * tanh(u)), u = 0.79788456 * (x + 0.044715 x^3)   (epilogues.cuh:22-44)
+    // With tanh(u) = 1 - 2 / (exp(2u) + 1) this is x - x / (exp(2u) + 1): one hardware exp2 and one hardware
+    // reciprocal (1 ulp each), safe at both ends (exp2 -> inf gives x, exp2 -> 0 gives 0).
+    constexpr float C1 = 2.0f * 0.79788456f * 1.4426950408889634f, C2 = C1 * 0.044715f;  // 2u * log2(e) = x (C1 + C2 x^2)
+    const float w = x * __builtin_fmaf(C2, x * x, C1);
+    const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(w) + 1.0f);
+    return __builtin_fmaf(-x, r, x);
 }
 
 // Partial sums of a tile shared by two workgroups travel through memory with system-scope accesses
