@@ -116,9 +116,6 @@ __device__ inline float4_t load_partial(__amdgpu_buffer_rsrc_t r, int tid, int q
 
 // NEXT: the epilogue also prepares the next layer's input (GELU, quantize, low-rank down); the plain
 // variant carries none of that code or of its registers.
-#ifndef SVDQ_ROPE_ENABLED
-#define SVDQ_ROPE_ENABLED true
-#endif
 template <bool ACT_UNSIGNED, bool FP4, bool NEXT>
 __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -800,7 +797,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (NEXT && SVDQ_ROPE_ENABLED && p.rotary && wcol0 < p.rope_cols) {
+        if (NEXT && p.rotary && wcol0 < p.rope_cols) {
             // EpilogueRMSNormRope (epilogues.cuh:269-425): the wave's 128 columns are one head of q or k.
             // The lane holds 64 values of its row, lane ^ 32 the other 64.  The (sin, cos) table is stored in
             // this loop's order ([32-row block][nt][q][lane] x float4: a wave-wide request is 1 KB
