@@ -153,7 +153,8 @@ typedef struct svdq_gemm_args {
     int64_t R_up, R_down;
     float alpha;            /* per-tensor scale (NVFP4 wtscale); must be 1 for INT4                 */
     int32_t act_unsigned;   /* INT4 activations are unsigned codes 0..15                            */
-    int32_t fuse_silu;      /* must be 0 (not implemented)                                          */
+    int32_t fuse_silu;      /* x * sigmoid(x) before the store (EpilogueSilu, gemm_base.cuh:783-792);
+                               only with `out` alone, as in launch_impl.cuh:404-417                  */
     int32_t fp4;            /* operands are NVFP4                                                   */
     /* RMS norm + rotary embedding of the q and k thirds of a fused QKV projection (all NULL / 0
      * otherwise).  Replaces EpilogueRMSNormRope, src/kernels/zgemm/epilogues.cuh:269-425, composed as in

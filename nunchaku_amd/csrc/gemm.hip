@@ -99,7 +99,8 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     SVDQ_REQUIRE(a->M_pad * a->N < (1ll << 40) && a->K < (1 << 24), "gemm: shape too large");
     // scale tables are addressed with 32-bit lane offsets
     SVDQ_REQUIRE((a->K / 64) * a->M_pad * 4 < (1ll << 31) && (a->K / 64) * a->N * 8 < (1ll << 31), "gemm: scale tables too large");
-    if (a->fuse_silu) return fail(SVDQ_EUNSUPPORTED, "gemm: fuse_silu is not implemented");
+    // SiLU goes with the plain store only (gemm_w4a4_launch_impl.cuh:404-417)
+    if (a->fuse_silu && (a->qout || a->rotary_emb || !a->out)) return fail(SVDQ_EUNSUPPORTED, "gemm: fuse_silu goes with `out` alone (no qout, no rotary_emb)");
     if (a->fp4 && a->act_unsigned) return fail(SVDQ_EINVAL, "gemm: NVFP4 activations are never unsigned");
     // INT4 adds the low-rank projection before scaling, which is exact only for power-of-two column factors
     // (the reference asserts alpha == 1 for INT4, gemm_w4a4_launch_impl.cuh:107, and only NVFP4 layers carry wcscales)
@@ -158,6 +159,7 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     p.rot_rows = (int)a->rot_rows;
     p.rope_cols = (int)(a->N / 3 * 2);
     p.norm_eps = a->norm_eps;
+    p.silu = a->fuse_silu != 0;
     p.gelu = a->qout != nullptr;  // the GELU is composed exactly when the next layer's input is produced (launch_impl.cuh:282-309)
 #ifdef SVDQ_GEMM_TIMING
     p.next_down = nullptr; p.next_lora_out = nullptr; p.R_down = 0;
@@ -195,7 +197,7 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
         p.partials = (float *)(w->ptr + w->counters_bytes);
     }
     // (the kernels with the next-layer epilogue also carry the norm + rotary epilogue)
-    const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr;
+    const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu;
     if (p.next_lora_out) {  // the low-rank projection for the next layer is accumulated across column blocks
         const int64_t n = a->M_pad * a->R_down;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, p.next_lora_out, n);

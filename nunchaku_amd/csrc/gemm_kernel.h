@@ -839,6 +839,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 }
             }
         }
+        if (NEXT && p.silu) {
+            // EpilogueSilu (gemm_base.cuh:783-792, gemm_utils.cuh:322-327): x * sigmoid(x) = x / (1 + exp(-x))
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    v[nt][e] = v[nt][e] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v[nt][e]));
+        }
         if (NEXT && p.gelu) {
 #pragma unroll
             for (int nt = 0; nt < 4; nt++)

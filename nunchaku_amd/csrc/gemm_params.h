@@ -51,6 +51,7 @@ struct GemmParams {
     float alpha;
     float lora_scales[8];
     int gelu;
+    int silu;  // x * sigmoid(x) before the store (next-layer variants only)
     // RMS norm + rotary embedding on the q and k heads of a fused QKV projection (next-layer variants only)
     const uint16_t *norm_q, *norm_k;  // bf16 [128]
     const float *rotary;              // fp32 [rot_rows/32][16][64 lanes][4], see svdq_gemm_args; null: no such epilogue

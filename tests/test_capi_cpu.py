@@ -79,7 +79,10 @@ def test_gemm_rejects_bad_arguments(lib):
     bad.M_out = 300
     assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
     bad = nv.GemmArgs.from_buffer_copy(a)
-    bad.fuse_silu = 1
+    bad.fuse_silu = 1  # only with `out` alone
+    bad.qout = 16
+    bad.oscales = 16
+    bad.next_smooth_rcp = 16
     assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
     # INT4 takes neither a per-tensor scale nor per-channel scales (NVFP4 only)
     bad = nv.GemmArgs.from_buffer_copy(a)

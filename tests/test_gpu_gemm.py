@@ -136,3 +136,27 @@ def test_gemm_unsupported_raises(dev):
     z = torch.zeros(256, 64, dtype=torch.uint8, device=dev)
     with pytest.raises(NotImplementedError):
         svdq_gemm_w4a4(act=z, wgt=z.view(torch.int8), ascales=z, wscales=z, out=z, poolout=z)
+
+
+def test_fuse_silu_epilogue(dev):
+    """fuse_silu: x * sigmoid(x) after bias and low-rank up, before the store (EpilogueSilu with
+    EpilogueDefault, gemm_w4a4_launch_impl.cuh:404-417)."""
+    from nunchaku_amd.ops import svdq_gemm_w4a4
+
+    M, K, N, R = 300, 256, 384, 32
+    announce(f"gemm fuse_silu M={M} K={K} N={N}")
+    layer = synth.make_layer(N, K, R, seed=61)
+    x = synth.make_activations(M, K, seed=61)
+    m = make_module(layer, dev)
+    ref = make_oracle(layer)
+    qx, asc, la = m.quantize(x.to(dev))
+    t = m.native_tensors()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    svdq_gemm_w4a4(act=qx, wgt=t["qweight"], out=out, ascales=asc, wscales=t["wscales"], lora_act_in=la, lora_up=t["proj_up"],
+                   bias=t["bias"], fuse_silu=True)
+    torch.cuda.synchronize()
+    codes, scales, lora = ref.quantize(x)
+    want = olin.gemm_w4a4(quant.dequant_int4(codes, scales), ref.w_deq, bias=ref.bias, lora_act_in=lora, lora_up=ref.proj_up, silu=True)[:M]
+    check_output(out, want)
+    plain = m.forward_quant(qx, asc, la)[:M]  # not the identity: the plain output differs
+    assert not torch.equal(plain, out)
