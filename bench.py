@@ -98,11 +98,12 @@ def main():
     ap.add_argument("--qkv-rope", action="store_true",
                     help="time the GEMM with the RMS-norm + rotary epilogue of fused_qkv_norm_rottary (workload flux_qkv); "
                          "the CPU comparison is skipped")
-    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "mfma-rate", "awq-gemv"], default=None,
+    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "mfma-rate", "awq-gemv", "fused-mlp"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
                          "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters; "
                          "'mfma-rate' measures the MFMA instruction of the GEMM alone; "
-                         "'awq-gemv' times the AWQ W4A16 GEMV at the modulation shape (1 row, K=3072, N=18432)")
+                         "'awq-gemv' times the AWQ W4A16 GEMV at the modulation shape (1 row, K=3072, N=18432); "
+                         "'fused-mlp' times fused_gelu_mlp on the FLUX MLP pair (M=4608, 3072 -> 12288 -> 3072)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -113,6 +114,31 @@ def main():
     if args.only == "mfma-rate":
         torch.cuda.init()
         print(f"mfma-rate: v_mfma_f32_32x32x16_f16 alone, TFLOP/s: {mfma_rate_probe()}")
+        return
+    if args.only == "fused-mlp":
+        from nunchaku_amd.models.linear import SVDQW4A4Linear
+        from nunchaku_amd.ops import fused_gelu_mlp
+        from oracle import synth
+
+        dev = torch.device("cuda:0")
+        M, K, N, R = 4608, 3072, 12288, 32
+        mods = []
+        for (n, k, unsigned, seed) in ((N, K, False, 2), (K, N, True, 3)):
+            mod = SVDQW4A4Linear(k, n, rank=R, act_unsigned=unsigned, device=dev)
+            mod.load_state_dict(synth.to_reference_checkpoint(synth.make_layer(n, k, R, seed=seed)))
+            mod.native_tensors()
+            mods.append(mod)
+        x = synth.make_activations(M, K, seed=2).to(dev).view(1, M, K)
+        for _ in range(20):
+            fused_gelu_mlp(x, mods[0], mods[1])
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fused_gelu_mlp(x, mods[0], mods[1])
+        e1.record()
+        torch.cuda.synchronize()
+        print(f"fused-mlp M={M} {K}->{N}->{K} rank {R}: {e0.elapsed_time(e1) * 1e3 / args.steps:.1f} us per call "
+              "(quantize + fc1 with GELU / next-layer quantize / low-rank-down epilogue + fc2)")
         return
     if args.only == "awq-gemv":
         from nunchaku_amd.ops import awq_gemv_w4a16
