@@ -54,6 +54,16 @@ def test_int4_no_smooth_and_padding_rows(dev):
     assert (codes[M:] == 0).all() and (osc.float()[:, M:] == 0).all() and (la[M:] == 0).all()
 
 
+@pytest.mark.parametrize("fp4", [False, True])
+def test_long_k_reads_smoothing_factors_from_global_memory(dev, fp4):
+    """K = 16512 (129 chunks, an odd count, 66 KB of reciprocal factors): beyond what the kernel keeps in LDS."""
+    M, K, R = 40, 16512, 32
+    announce(f"quantize long K M={M} K={K} fp4={fp4}")
+    layer = synth.make_layer(128, K, R, seed=5, fp4=fp4)
+    x = synth.make_activations(M, K, seed=5)
+    _check(x, layer, *_run(dev, x, layer, fp4=fp4), fp4=fp4)
+
+
 def test_int4_edge_values(dev):
     # zero groups, negative zero, exact .5 ties of the smoothing quotient, huge and tiny magnitudes
     M, K, R = 256, 256, 16
