@@ -892,15 +892,25 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             // lora.cuh:243-353): this wave's 128 columns are one 128-chunk of the next layer's K
             const int RT = p.R_down / 16;
             const int r16 = lane & 15, q = lane >> 4;
+            // (the operands of rank tile rt + 1 are requested before rank tile rt is worked on: one exposed
+            // memory latency per slab instead of one per rank tile)
+            bf16x8_t nb[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) nb[i] = p.next_down[((size_t)((wcol0 / 128) * 4 + i) * RT) * 64 + lane];
             for (int rt = 0; rt < RT; rt++) {
                 float4_t d[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+                bf16x8_t b[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) b[i] = nb[i];
+                const int rt_next = rt + 1 < RT ? rt + 1 : rt;
+#pragma unroll
+                for (int i = 0; i < 4; i++) nb[i] = p.next_down[((size_t)((wcol0 / 128) * 4 + i) * RT + rt_next) * 64 + lane];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const bf16x8_t b = p.next_down[((size_t)((wcol0 / 128) * 4 + i) * RT + rt) * 64 + lane];
 #pragma unroll
                     for (int m2 = 0; m2 < 2; m2++) {
                         const bf16x8_t a = *(const bf16x8_t *)(slab + (16 * m2 + r16) * OUT_LD + 32 * q + 8 * i);
-                        d[m2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, d[m2], 0, 0, 0);
+                        d[m2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[i], d[m2], 0, 0, 0);
                     }
                 }
 #pragma unroll
