@@ -36,8 +36,7 @@ WORKLOADS = {
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, the peak the metric is quoted against
 # HBM-side bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
 # read for a device copy of known size (profiles/hbm_traffic_*.md); only known for the profiled workload
-PROFILED_GEMM_TRAFFIC_BYTES = {"flux_mlp_fc1": (2.0 * 212654 + 1.0 * 193586) * 1024}
-FP16_PEAK_TFLOPS = 2500.0
+PROFILED_GEMM_TRAFFIC_BYTES = {}
 HBM_PEAK_GBS = 8000.0
 
 
@@ -67,26 +66,6 @@ def cpu_baseline(layer, x, rows: int, iters: int = 20):
     }, y
 
 
-def mfma_rate_probe():
-    """Sustained rate of the GEMM's own MFMA instruction in a loop of nothing else (TFLOP/s), with constant
-    and with random operand bits; None if the probe library has not been built."""
-    import ctypes
-
-    from nunchaku_amd import _native as nv
-
-    if not nv.PROBE_LIB_PATH.exists():
-        return None
-    lib = ctypes.CDLL(str(nv.PROBE_LIB_PATH))
-    lib.svdq_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
-    res = {}
-    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
-        v = ctypes.c_double(0.0)
-        if lib.svdq_probe_mfma_rate(rnd, 20000, 10, ctypes.byref(v)) != 0:
-            return None
-        res[name] = v.value
-    return res
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,10 +77,9 @@ def main():
     ap.add_argument("--qkv-rope", action="store_true",
                     help="time the GEMM with the RMS-norm + rotary epilogue of fused_qkv_norm_rottary (workload flux_qkv); "
                          "the CPU comparison is skipped")
-    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "mfma-rate", "awq-gemv", "fused-mlp"], default=None,
+    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "awq-gemv", "fused-mlp"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
                          "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters; "
-                         "'mfma-rate' measures the MFMA instruction of the GEMM alone; "
                          "'awq-gemv' times the AWQ W4A16 GEMV at the modulation shape (1 row, K=3072, N=18432); "
                          "'fused-mlp' times fused_gelu_mlp on the FLUX MLP pair (M=4608, 3072 -> 12288 -> 3072)")
     args = ap.parse_args()
@@ -111,10 +89,6 @@ def main():
 
     import torch
 
-    if args.only == "mfma-rate":
-        torch.cuda.init()
-        print(f"mfma-rate: v_mfma_f32_32x32x16_f16 alone, TFLOP/s: {mfma_rate_probe()}")
-        return
     if args.only == "fused-mlp":
         from nunchaku_amd.models.linear import SVDQW4A4Linear
         from nunchaku_amd.ops import fused_gelu_mlp
@@ -188,7 +162,9 @@ def main():
     xd = x.to(dev)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     M_pad = (M + 255) // 256 * 256
-    qx = torch.empty(M_pad, K // 2, dtype=torch.uint8, device=dev)
+    from nunchaku_amd import packing
+
+    qx = torch.empty(M_pad, packing.act_nbytes_per_row(K, fp4), dtype=torch.uint8, device=dev)
     asc = torch.empty(K // 16, M_pad, dtype=torch.float8_e4m3fn, device=dev) if fp4 else torch.empty(K // 64, M_pad, dtype=torch.bfloat16, device=dev)
     la = torch.empty(M_pad, R, dtype=torch.float32, device=dev)
     t = mod.native_tensors()
@@ -240,6 +216,14 @@ def main():
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    # the same loop timed by events on the launch stream: what the GPU spent, without the host's share
+    s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s0.record()
+    for _ in range(args.steps):
+        step()
+    s1.record()
+    torch.cuda.synchronize()
+    ms_per_step_events = s0.elapsed_time(s1) / args.steps
 
     # per-kernel durations with events on the stream the kernels are launched on
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
@@ -271,12 +255,13 @@ def main():
         "metric": "effective TOPS of fused W4A4+LoRA linear at FLUX M=4608; % of MFMA peak",
         "value": value, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16" if fp4 else "e2m3 x e2m3 -> f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: SVDQW4A4Linear forward M={M} K={K} N={N} rank={R} {'NVFP4 g16' if fp4 else 'INT4 g64'} bf16 in/out"
                                + (" + RMS norm and rotary embedding on q, k in the GEMM epilogue" if args.qkv_rope else ""),
                    "M": M, "K": K, "N": N, "rank": R},
         "pct_of_int8_mfma_peak": 100.0 * value / INT8_PEAK_TOPS,
         "us_per_layer": ms_per_step * 1e3,
+        "us_per_layer_events": ms_per_step_events * 1e3,
         "kernels": {
             "quantize_fuse_lora_us": tq_us, "gemm_us": tg_us, "quantize_fuse_lora_us_back_to_back": tq_b2b_us,
             "quantize_GBps": bytes_quant / (tq_b2b_us * 1e-6) / 1e9,
@@ -284,13 +269,11 @@ def main():
             "gemm_main_term_TOPS": 2.0 * M * N * K / (tg_us * 1e-6) / 1e12,
         },
         "roofline": {
-            "kernel": f"gemm_w4a4_kernel<false, {'true' if fp4 else 'false'}, {'true' if args.qkv_rope else 'false'}>", "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
+            "kernel": (f"gemm_w4a4_kernel<{'true' if args.qkv_rope else 'false'}>" if fp4 else f"g6::gemm6_kernel<{'true' if args.qkv_rope else 'false'}>"),
+            "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
             "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": PROFILED_GEMM_TRAFFIC_BYTES.get(args.workload),
-            "peak_basis": "dense INT8 MFMA (the metric's peak); the kernel issues fp16 MFMA, dense peak 2500",
-            "frac_of_fp16_mfma_peak": gemm_tops / FP16_PEAK_TFLOPS,
-            # what this GPU sustains on the same instruction with no other work (probe_mfma_rate.hip): with
-            # random operand bits the power management lowers the clock, as it does under the GEMM
-            "fp16_mfma_alone_tflops": mfma_rate_probe(),
+            "peak_basis": "dense INT8 MFMA (the metric's peak)" + ("; the NVFP4 kernel issues fp16 MFMA, dense peak 2500" if fp4 else
+                          "; the INT4 kernel issues one fp6 MFMA (dense peak 10100) and one small bf16 MFMA per 32x32 tile and k-group"),
         },
     }
     if not args.no_cpu:

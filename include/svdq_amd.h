@@ -10,13 +10,20 @@
  *   - plain pointers to DEVICE memory, sizes as int64_t, no framework types;
  *   - every function only enqueues work on `stream` (a hipStream_t passed as void*) and returns;
  *     no synchronisation; safe to call from several threads.  One exception to "no allocation, no
- *     global state": svdq_gemm_w4a4 keeps one workspace per (device, stream) pair, see there;
+ *     global state": some calls of svdq_gemm_w4a4 keep a workspace per (device, stream) pair, see there;
  *   - return value 0 on success, a negative SVDQ_E* code otherwise; arguments are validated before
  *     anything is launched, so a failed call has no side effect;
  *   - `svdq_last_error()` returns a thread-local human-readable message for the last failure.
  *
  * Notation: M tokens, M_pad = M rounded up to 256, K in-features, N out-features, R low-rank rank,
  * G group size (64 for INT4, 16 for NVFP4).
+ *
+ * INT4 operands (activations and weights alike) are held as E2M3 (fp6) patterns of code / 2 -- exact
+ * for every code in [-8, 15] -- in "fragments": one operand of the fp6 matrix instruction, 32 rows x
+ * one 64-wide k-group = 1536 bytes.  Slot s = row + 32 * half (half: which 32 of the 64 codes) owns a
+ * 192-bit string, code j of its half in bits [6 j, 6 j + 6); the first 16 bytes of the string lie at
+ * byte 16 s of the fragment, the last 8 at 1024 + 8 s.  Activations: [M_pad/128][K/64][4 fragments]
+ * (0.75 byte per element); weights: [ceil(N/256)][K/64][8 fragments], columns beyond N zero.
  */
 #ifndef SVDQ_AMD_H
 #define SVDQ_AMD_H
@@ -32,7 +39,7 @@ extern "C" {
 #define SVDQ_EUNSUPPORTED -2 /* valid request that this build does not implement */
 #define SVDQ_ELAUNCH -3      /* the HIP runtime refused the launch */
 
-#define SVDQ_ABI_VERSION 2
+#define SVDQ_ABI_VERSION 3
 
 int svdq_abi_version(void);
 const char *svdq_last_error(void);
@@ -45,18 +52,17 @@ const char *svdq_last_error(void);
  * ------------------------------------------------------------------------------------------ */
 
 /* qweight int8 [N, K/2] (reference lane order, two's complement nibbles)
- *   -> native int8 [N, K/2]: tiles [N/32][K/64][32 rows][32 bytes], byte b of a (row, group) holds
- *      elements 2b (low nibble) and 2b+1 (high nibble).  INT4 codes are stored offset-binary
- *      (code + 8); NVFP4 patterns (fp4 != 0) are stored unchanged.
+ *   INT4 (fp4 == 0) -> E2M3 fragments [ceil(N/256)][K/64][8], ceil(N/256) * 256 * K * 3 / 4 bytes;
+ *   NVFP4 (fp4 != 0) -> int8 [N, K/2]: tiles [N/32][K/64][32 rows][32 bytes], byte b of a (row, group)
+ *      holds elements 2b (low nibble) and 2b+1 (high nibble), patterns unchanged.
  * Replaces the implicit layout contract of packed_wgt_t loads, gemm_base.cuh:278-294. */
 int svdq_repack_qweight(const void *src, void *dst, int64_t N, int64_t K, int fp4, void *stream);
 
-/* wscales bf16 [K/64, N] (reference lane order) -> native:
- *   dst_scales fp16 [K/64, N]  = wscales[g, n] * 2^e[n]   (column-normalised so that the largest
- *                               scale of a column lies in [2^11, 2^12); exact, power-of-two shift)
- *   dst_colnorm fp32 [N]       = 2^-e[n]
- * Replaces packed_wscale_t loads, gemm_base.cuh:474-489. */
-int svdq_repack_wscales(const void *src, void *dst_scales, void *dst_colnorm, int64_t N, int64_t K, void *stream);
+/* INT4 wscales bf16 [K/64, N] (reference lane order) -> native [ceil(N/256)][K/64][256 columns] x 8 bytes
+ * {bf16(4 * scale), 0, 0, 0}: the operand of the matrix instruction that forms the per-group factor
+ * (the 4 undoes the halving of both operands' codes; columns beyond N hold zero).
+ * ceil(N/256) * 256 * (K/64) * 8 bytes.  Replaces packed_wscale_t loads, gemm_base.cuh:474-489. */
+int svdq_repack_wscales(const void *src, void *dst_scales, int64_t N, int64_t K, void *stream);
 
 /* NVFP4 micro scales fp8-e4m3 [K/16, N] (reference lane order) -> native fp16 [K/64][N][4] (the four
  * 16-groups of a 64-wide k tile side by side) and fp32 colnorm [N], normalised as above.
@@ -91,8 +97,8 @@ int svdq_repack_rotemb(const void *src, void *dst, int64_t rows, void *stream);
  * ------------------------------------------------------------------------------------------ */
 typedef struct svdq_quantize_args {
     const void *input;      /* bf16 [M, K] row-major */
-    void *output;           /* u8 [M_pad, K/2] native activation tiles [M_pad/32][K/G64][32][32 B];
-                               INT4 codes offset-binary (code + 8), NVFP4 patterns unchanged      */
+    void *output;           /* INT4: E2M3 fragments [M_pad/128][K/64][4], M_pad * K * 3 / 4 bytes;
+                               NVFP4: u8 [M_pad, K/2] tiles [M_pad/32][K/64][32 rows][32 B]         */
     void *oscales;          /* INT4: bf16 [K/64][M_pad]; NVFP4: fp8-e4m3, K/16 * M_pad values stored as
                                [K/64][M_pad][4] (four 16-groups of a 64-group side by side)      */
     const void *lora_down;  /* native proj_down (svdq_repack_lora_down) or NULL when R == 0       */
@@ -113,45 +119,46 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  *   layer] -> store bf16 `out` and/or shift + smooth + quantize for the next layer (`qout`).
  * The GELU is applied exactly when `qout` is given (launch_impl.cuh:282-309).
  *
- * INT4 calls must have alpha == 1 and no wcscales (the reference asserts alpha == 1 for INT4,
- * launch_impl.cuh:107, and only NVFP4 layers carry wcscales): SVDQ_EUNSUPPORTED otherwise.
+ * INT4 runs on the fp6 matrix instruction (one workgroup per 128 x 256 output tile); NVFP4 runs on the
+ * fp16 matrix instruction with dequantized operands (persistent workgroups, 256 x 256 tiles).
  *
- * Workspace: the work is split evenly over one workgroup per compute unit, so an output tile can be
- * shared by two workgroups (by more when there are fewer tiles than compute units: the tiles are then
- * split along K), which exchange fp32 partial sums through device memory.  Unless the
- * number of 256x256 output tiles is a multiple of the number of compute units (or smaller), the
- * call needs a workspace of 512 KB per compute unit (128 MB on MI355X) plus 4 bytes per tile.  The
- * library allocates it with hipMalloc the first time a (device, stream) pair needs it (that call is
- * not capturable into a graph and may synchronise), keeps it until the process ends and reuses it
- * for every later call on that pair; at most 16 pairs.  Calls on one stream run in order and share
- * the workspace safely; the same stream must not be used from two threads at once.  Setting the
- * environment variable SVDQ_GEMM_NO_SHARED_TILES makes every call use whole tiles only (no workspace,
- * slower when the tile count does not divide evenly).  With fewer tiles than compute units a workgroup gets at least
- * 12 units (of 128 along K) of work; SVDQ_GEMM_MIN_UNITS overrides that number.
+ * Workspace.  Most INT4 calls need none and touch no global state.  Three kinds of call keep a
+ * workspace per (device, stream) pair, allocated with hipMalloc the first time the pair needs it (that
+ * call is not capturable into a graph and may synchronise), kept until the process ends, grown when a
+ * later call needs more (after a stream synchronisation), at most 16 pairs:
+ *   - INT4 with so few output tiles that they are split along K (fewer tiles than compute units, or
+ *     k_split > 1): 128 KB of fp32 partial sums per tile and part;
+ *   - INT4 with next_lora_down: 8 bytes per element of next_lora_act_out (fixed-point sums, which make
+ *     the result independent of the order in which the column blocks arrive);
+ *   - NVFP4 whenever the number of 256 x 256 tiles is not a multiple of the number of compute units:
+ *     512 KB per compute unit.
+ * Calls on one stream run in order and share the workspace safely; the same stream must not be used
+ * from two threads at once.  svdq_gemm_w4a4_noalloc is the variant for callers that cannot allocate.
  * ------------------------------------------------------------------------------------------ */
 typedef struct svdq_gemm_args {
-    const void *act;        /* u8 native activation tiles [M_pad, K/2]                              */
+    const void *act;        /* as written by operator 1 (INT4: E2M3 fragments; NVFP4: nibble tiles)     */
     const void *ascales;    /* as written by operator 1: bf16 [K/64][M_pad] or fp8 [K/64][M_pad][4] */
     const void *wgt;        /* native qweight (svdq_repack_qweight)                                 */
-    const void *wscales;    /* native fp16 scales (svdq_repack_wscales / _wmscales)                 */
-    const float *colnorm;   /* fp32 [N] from the same repack call                                   */
+    const void *wscales;    /* native scales (svdq_repack_wscales / _wmscales)                      */
+    const float *colnorm;   /* NVFP4: fp32 [N] from svdq_repack_wmscales; INT4: ignored, may be NULL */
     const void *bias;       /* bf16 [N] channel order, or NULL                                      */
-    const void *wcscales;   /* bf16 [N] channel order, or NULL; no element may be zero (the low-rank
-                               term is added in units of the column factor)                         */
+    const void *wcscales;   /* bf16 [N] channel order, or NULL; NVFP4: no element may be zero (the
+                               low-rank term is added in units of the column factor)                */
     const float *lora_act_in; /* fp32 [M_pad, R_up] row-major, or NULL                              */
     const void *lora_up;    /* bf16 [N, R_up] (svdq_repack_lora_up), or NULL                        */
     const float *lora_scales; /* HOST pointer, ceil(R_up/16) floats, or NULL for all ones           */
     void *out;              /* bf16 [M_out, N_out] row-major, or NULL                               */
     /* next-layer fusion (all NULL unless qout is given) */
-    void *qout;             /* u8 native activation tiles [M_pad, N/2] for the next layer           */
+    void *qout;             /* the next layer's activations, in operator 1's output format           */
     void *oscales;          /* bf16 [N/64][M_pad] (INT4 unsigned) or fp8 [N/64][M_pad][4] (NVFP4)   */
     const float *next_smooth_rcp; /* fp32 [N] from svdq_repack_smooth of the next layer             */
     const void *next_lora_down;   /* native proj_down of the next layer ([N, R_down]) or NULL       */
-    float *next_lora_act_out;     /* fp32 [M_pad, R_down]; zeroed and accumulated by the call       */
+    float *next_lora_act_out;     /* fp32 [M_pad, R_down]; fully written by the call                */
     int64_t M_pad, N, K;
     int64_t M_out, N_out;   /* shape of `out` (M_out <= M_pad, N_out <= N)                          */
     int64_t R_up, R_down;
-    float alpha;            /* per-tensor scale (NVFP4 wtscale); must be 1 for INT4                 */
+    float alpha;            /* per-tensor scale (NVFP4 wtscale; the reference asserts 1 for INT4,
+                               launch_impl.cuh:107, this library applies whatever is given)          */
     int32_t act_unsigned;   /* INT4 activations are unsigned codes 0..15                            */
     int32_t fuse_silu;      /* x * sigmoid(x) before the store (EpilogueSilu, gemm_base.cuh:783-792);
                                only with `out` alone, as in launch_impl.cuh:404-417                  */
@@ -170,6 +177,9 @@ typedef struct svdq_gemm_args {
                                (svdq_repack_rotemb writes it from the reference's pack_rotemb order)  */
     int64_t rot_rows;       /* rows of rotary_emb: M_out <= rot_rows <= M_pad, a multiple of 32      */
     float norm_eps;         /* the reference uses 1e-6 (launch_impl.cuh:374)                        */
+    int32_t k_split;        /* 0: the library decides.  n > 0: split every output tile along K into n parts
+                               whose partial sums meet in the workspace (1: never split); a tuning and
+                               testing knob with no counterpart in the reference                      */
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);

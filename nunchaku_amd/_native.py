@@ -18,14 +18,13 @@ import torch
 _PKG_DIR = Path(__file__).resolve().parent
 _CSRC = _PKG_DIR / "csrc"
 LIB_PATH = _PKG_DIR / "libsvdq_amd.so"
-PROBE_LIB_PATH = _PKG_DIR / "libsvdq_probe.so"  # bench.py's MFMA-rate probe (csrc/probe_mfma_rate.hip)
 SOURCES = ["repack.hip", "quantize.hip", "gemm.hip", "awq_gemv.hip"]
 HIPCC_FLAGS = [
     "-shared", "-fPIC", "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
-SVDQ_ABI_VERSION = 2
+SVDQ_ABI_VERSION = 3
 EXPORTED_SYMBOLS = [
     "svdq_abi_version", "svdq_last_error",
     "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
@@ -61,7 +60,7 @@ class GemmArgs(ctypes.Structure):
         ("alpha", ctypes.c_float), ("act_unsigned", ctypes.c_int32), ("fuse_silu", ctypes.c_int32),
         ("fp4", ctypes.c_int32),
         ("norm_q", ctypes.c_void_p), ("norm_k", ctypes.c_void_p), ("rotary_emb", ctypes.c_void_p),
-        ("rot_rows", ctypes.c_int64), ("norm_eps", ctypes.c_float),
+        ("rot_rows", ctypes.c_int64), ("norm_eps", ctypes.c_float), ("k_split", ctypes.c_int32),
     ]
 
 
@@ -75,7 +74,9 @@ class AwqGemvArgs(ctypes.Structure):
     ]
 
 
-GEMM_VARIANTS = 6  # gemm_variant.hip is compiled once per kernel variant (-DSVDQ_VARIANT=n)
+# kernel variants, one translation unit each (-DSVDQ_VARIANT=n): the INT4 GEMM (gemm6_variant.hip: plain /
+# next-layer epilogue) and the NVFP4 GEMM (gemm_variant.hip: the same two)
+GEMM_VARIANT_UNITS = [("gemm6_variant.hip", 0), ("gemm6_variant.hip", 1), ("gemm_variant.hip", 4), ("gemm_variant.hip", 5)]
 
 
 def build(verbose: bool = False, extra_flags: tuple[str, ...] = (), lib_path: Path | None = None) -> Path:
@@ -89,7 +90,7 @@ def build(verbose: bool = False, extra_flags: tuple[str, ...] = (), lib_path: Pa
     out = Path(lib_path) if lib_path else LIB_PATH
     with tempfile.TemporaryDirectory(prefix="svdq_build_") as tmp:
         jobs = [([str(_CSRC / src)], Path(tmp) / (src + ".o")) for src in SOURCES]
-        jobs += [([str(_CSRC / "gemm_variant.hip"), f"-DSVDQ_VARIANT={v}"], Path(tmp) / f"gemm_variant_{v}.o") for v in range(GEMM_VARIANTS)]
+        jobs += [([str(_CSRC / src), f"-DSVDQ_VARIANT={v}"], Path(tmp) / f"{src}_{v}.o") for src, v in GEMM_VARIANT_UNITS]
 
         def compile_one(job):
             args, obj = job
@@ -104,11 +105,6 @@ def build(verbose: bool = False, extra_flags: tuple[str, ...] = (), lib_path: Pa
                               capture_output=True, text=True)
         if link.returncode != 0:
             raise RuntimeError("hipcc link failed:\n" + link.stderr[-4000:])
-        if lib_path is None:
-            # measurement aid of bench.py, a library of its own: not part of the operator ABI
-            probe = subprocess.run([hipcc, *HIPCC_FLAGS, str(_CSRC / "probe_mfma_rate.hip"), "-o", str(PROBE_LIB_PATH)], capture_output=True, text=True)
-            if probe.returncode != 0:
-                raise RuntimeError("hipcc failed on probe_mfma_rate.hip:\n" + probe.stderr[-4000:])
     if verbose:
         print(f"built {out}")
     return out
@@ -131,7 +127,7 @@ def lib() -> ctypes.CDLL:
         L.svdq_last_error.restype = ctypes.c_char_p
         i64, vp, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
         L.svdq_repack_qweight.argtypes = [vp, vp, i64, i64, ci, vp]
-        L.svdq_repack_wscales.argtypes = [vp, vp, vp, i64, i64, vp]
+        L.svdq_repack_wscales.argtypes = [vp, vp, i64, i64, vp]
         L.svdq_repack_wmscales.argtypes = [vp, vp, vp, i64, i64, vp]
         L.svdq_repack_vector.argtypes = [vp, vp, i64, vp]
         L.svdq_repack_smooth.argtypes = [vp, vp, i64, vp]

@@ -1,32 +1,27 @@
-// Operator 2: W4A4 GEMM with fused epilogue for gfx950.  Counterpart of gemm_w4a4_kernel /
-// gemm_w4a4_fp4_kernel (src/kernels/zgemm/gemm_w4a4.cuh:1046-1095, :358-405) and of the epilogue
-// chain composed in gemm_w4a4_launch_impl.cuh:172-309.
+// Operator 2, NVFP4 operands: W4A4 GEMM with fused epilogue for gfx950.  Counterpart of
+// gemm_w4a4_fp4_kernel (src/kernels/zgemm/gemm_w4a4.cuh:273-405) and of the epilogue chain composed in
+// gemm_w4a4_launch_impl.cuh:172-309.  (INT4 operands take gemm6_kernel.h.)
 //
 // How the contraction is mapped to the matrix cores
 // -------------------------------------------------
-// Every 64-wide (16-wide for NVFP4) k-group carries its own activation scale (per row) and weight
-// scale (per column).  Applying them after an integer MFMA costs three VALU instructions per
-// accumulator per group, which caps an int8-MFMA kernel far below the matrix-core rate.  Instead
-// both operands are dequantized *in registers* to fp16 -- (code) * (scale) is exact in fp16 because
-// a 4-bit code has at most 3 significant bits and a bf16 / e4m3 scale at most 8 -- and fed to
-// v_mfma_f32_32x32x16_f16 with fp32 accumulation.  The result equals the fp32 dequantize-then-matmul
-// definition up to fp32 summation order; no per-group post-scaling exists.
+// Every 16-wide k-group carries its own activation scale (per row, E4M3) and weight scale (per column,
+// E4M3).  The block-scaled fp4 matrix instruction takes power-of-two scales per 32 elements only, so
+// both operands are dequantized *in registers* to fp16 -- (code) * (scale) is exact in fp16: an E2M1
+// code has 2 significant bits and an E4M3 scale 4 -- and fed to v_mfma_f32_32x32x16_f16 with fp32
+// accumulation.  The result equals the fp32 dequantize-then-matmul definition up to fp32 summation
+// order; no per-group post-scaling exists.
 //
 // Range: activation scales are renormalised per row and weight scales per column by powers of two
 // (largest scale of a row / column moved into [2^10, 2^11)), so the fp16 products never overflow and
 // only contributions 2^-25 below the largest of their row / column can underflow.  The shifts are
 // undone exactly in the epilogue.
 //
-// Dequantization of one INT4 word (8 codes; the nibble word is stored rotated left by 2 bits so that
-// two codes sit on fp16 mantissa bits [9:6] of the two halves, the other pairs a shift / rotate away):
-//   (w' & 0x03C003C0) | 0x3C003C00 -> two fp16 values 1 + u/16,  w' in {w, w >> 4, w << 4, rotl(w, 8)}
-//   packed fma with (16 s, -24 s)   -> (u - 8) s, exact (offset-binary signed codes; -16 s: unsigned)
-// = 11 VALU instructions per 8 codes.  Both operands use the same element-to-slot order, so the
-// contraction pairs equal k.  NVFP4 words use the hardware E2M1 -> fp16 conversion and one packed
-// multiply per pair (8 instructions per 8 codes).
+// Dequantization of one word (8 E2M1 patterns): the hardware E2M1 -> fp16 conversion and one packed
+// multiply per pair (8 instructions per 8 codes).  Both operands use the same element-to-slot order, so
+// the contraction pairs equal k.
 //
 // Tiling: workgroup = 4 waves (2 x 2), block tile 256 x 256, wave tile 128 x 128 = 4 x 4 MFMA tiles,
-// 256 fp32 accumulators per lane.  Operand tiles are staged through a 3-deep LDS ring, one k-group
+// 256 fp32 accumulators per lane.  Operand tiles are staged through a 4-deep LDS ring, one k-group
 // per stage; global loads for group g+3 are issued before the math of group g.
 #pragma once
 
@@ -37,39 +32,9 @@
 
 namespace svdq {
 
-#ifdef SVDQ_GEMM_TIMING
-#define SVDQ_STAMP(i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 64 + (i)] = __builtin_readcyclecounter()
-#define SVDQ_STAMP_TILE(t, i) if (p.stamps && threadIdx.x == 0) p.stamps[blockIdx.x * 64 + 8 + (t) * 8 + (i)] = __builtin_readcyclecounter()
-#else
-#define SVDQ_STAMP(i)
-#define SVDQ_STAMP_TILE(t, i)
-#endif
-
-
 
 __device__ inline half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 __device__ inline uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
-
-struct DequantConsts {
-    uint32_t magic;  // fp16 pair 1.0: OR-ing a code into mantissa bits [9:6] gives 1 + u/16
-    uint32_t mask;   // 0x03C003C0; kept opaque so that (w & mask) | magic becomes one v_and_or_b32
-};
-
-// 8 INT4 codes of one (rotated) word -> 8 fp16 values (code - bias) * scale.  `mul` = 16 * scale and
-// `add` = -(16 + bias) * scale as fp16 pairs (bias 8 for offset-binary signed codes, 0 for unsigned):
-// fma(1 + u/16, 16 s, -(16 + bias) s) = (u - bias) s with a single, exact rounding.
-// Slot order (identical for both operands): elements [1,5,2,6,0,4,7,3].
-__device__ inline half8_t dequant_word(uint32_t w, half2_t mul, half2_t add, const DequantConsts &dc) {
-    const half2_t t0 = as_half2((w & dc.mask) | dc.magic);
-    const half2_t t1 = as_half2(((w >> 4) & dc.mask) | dc.magic);
-    const half2_t t2 = as_half2(((w << 4) & dc.mask) | dc.magic);
-    const half2_t t3 = as_half2((__builtin_amdgcn_alignbit(w, w, 24) & dc.mask) | dc.magic);
-    const half2_t a0 = __builtin_elementwise_fma(t0, mul, add);
-    const half2_t a1 = __builtin_elementwise_fma(t1, mul, add);
-    const half2_t a2 = __builtin_elementwise_fma(t2, mul, add);
-    const half2_t a3 = __builtin_elementwise_fma(t3, mul, add);
-    return half8_t{a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
-}
 
 // 8 E2M1 patterns of one word -> 8 fp16 values pattern_value * scale, slot order [0..7].  The
 // hardware conversion yields the exact E2M1 value (its scale operand only contributes an exponent).
@@ -116,7 +81,7 @@ __device__ inline float4_t load_partial(__amdgpu_buffer_rsrc_t r, int tid, int q
 
 // NEXT: the epilogue also prepares the next layer's input (GELU, quantize, low-rank down); the plain
 // variant carries none of that code or of its registers.
-template <bool ACT_UNSIGNED, bool FP4, bool NEXT>
+template <bool NEXT>
 __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // Thread coordinates.  They are re-derived from an opaque copy of the thread index at the top of every
@@ -127,14 +92,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     int wm = wave >> 1, wn = wave & 1;
     int r32 = lane & 31, h = lane >> 5;
     int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
-    uint32_t code_voff = lane * 16, as_voff = lane * (FP4 ? 4 : 2);  // (the wave's part of the scale offset is in as_base)
+    uint32_t code_voff = lane * 16, as_voff = lane * 4;  // (the wave's part of the scale offset is in as_base)
     auto refresh_thread_coordinates = [&]() {
         int t = threadIdx.x;
         asm volatile("" : "+v"(t));
         tid = t; lane = t & 63; wave = t >> 6;
         wm = wave >> 1; wn = wave & 1; r32 = lane & 31; h = lane >> 5;
         ca = __builtin_amdgcn_readfirstlane(t >> 6);
-        code_voff = lane * 16; as_voff = lane * (FP4 ? 4 : 2);
+        code_voff = lane * 16; as_voff = lane * 4;
     };
 
     // ---- persistent workgroups, work split in units of two k-groups ----------------------------
@@ -175,7 +140,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         hi = (int)((t1 * nwg - 1) / units);                    // last v with units v / nwg < t1
     };
     int *rowshift = (int *)(lds + SHIFT_OFF);  // [MAX_BATCH][256] power-of-two renormalisation of the rows
-    constexpr uint32_t AS_ELT = FP4 ? 4 : 2, BS_ELT = FP4 ? 8 : 2;  // bytes of scales per (64-group, row / column)
+    constexpr uint32_t AS_ELT = 4, BS_ELT = 8;  // bytes of scales per (64-group, row / column)
     const uint32_t as_stride = (uint32_t)p.M_pad * AS_ELT, bs_stride = (uint32_t)p.N * BS_ELT;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
 
@@ -215,8 +180,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             c.a_base[j] = p.act + (size_t)(c.m0 / 32 + t) * kgroups * TILE_BYTES;
             c.b_base[j] = p.wgt + (size_t)tb * kgroups * TILE_BYTES;
         }
-        // scale sources: INT4 one bf16 / fp16 value per (group, row / column); NVFP4 one word of four
-        // e4m3 (activations) or four fp16 (weights) per (64-group, row / column)
+        // scale sources: one word of four e4m3 (activations) or four fp16 (weights) per (64-group, row / column)
         c.as_base = (const uint8_t *)p.ascales + (size_t)(c.m0 + ca * 64) * AS_ELT;  // row m0 + tid = m0 + 64 ca + lane
         // column n0 + tid = n0 + 64 ca + lane; a wave beyond N reads the last 64 columns instead (its scales are
         // stored as zero), so that the lane part of the offset is the same everywhere and needs no register
@@ -249,62 +213,30 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                          :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(voff), "s"(c.b_base[j]) : "memory");
         }
     };
+    // (ordinary loads: the compiler tracks the registers they write and places the waits for them itself.
+    // They are issued AFTER the asynchronous copies of the same groups, which the compiler does not count:
+    // its "all but the n newest requests" waits then cover the older copies too and never wait for less
+    // than intended.)
     auto issue_scales = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
         const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
-        // (the lane's scale offset is derived from the live code offset on the spot: one shift, and no
-        // register of its own across the loop)
-        uint32_t lane_off;
-        if (!FP4)
-            asm volatile("v_lshrrev_b32 %0, 3, %1" : "=v"(lane_off) : "v"(code_voff));
-        else
-            asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(lane_off) : "v"(code_voff));
-        uint32_t lane_off_b;
-        if (!FP4)
-            asm volatile("v_lshrrev_b32 %0, 3, %1" : "=v"(lane_off_b) : "v"(code_voff));
-        else
-            asm volatile("v_lshrrev_b32 %0, 1, %1" : "=v"(lane_off_b) : "v"(code_voff));
-        const uint32_t va = (uint32_t)gc * as_stride + lane_off, vb = (uint32_t)gc * bs_stride + lane_off_b;
-        if (!FP4) {
-            uint32_t t;
-            asm volatile("global_load_ushort %0, %1, %2" : "=v"(ra) : "v"(va), "s"(c.as_base) : "memory");
-            asm volatile("global_load_ushort %0, %1, %2" : "=v"(t) : "v"(vb), "s"(c.bs_base) : "memory");
-            rb[0] = t;
-        } else {
-            asm volatile("global_load_dword %0, %1, %2" : "=v"(ra) : "v"(va), "s"(c.as_base) : "memory");
-            asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(rb) : "v"(vb), "s"(c.bs_base) : "memory");
-        }
+        ra = *(const uint32_t *)(c.as_base + ((uint32_t)gc * as_stride + as_voff));
+        rb = *(const u32x2_t *)(c.bs_base + ((uint32_t)gc * bs_stride + as_voff * 2));
     };
     auto store_scales = [&](const TileCtx &c, int g, uint32_t ra, u32x2_t rb) {
         // (row / column tid of the stage tables, addressed through the lane offset that is live anyway:
         // the main loop has no register to spare for another address)
         uint8_t *base = lds + (g % STAGES) * STAGE_BYTES + ca * 1024 + code_voff;
-        if (!FP4) {
-            const _Float16 sa = (_Float16)ldexpf(bf16_bits_to_f32(ra & 0xFFFFu), c.shift);
-            const _Float16 sb = c.col_ok ? __builtin_bit_cast(_Float16, (uint16_t)rb[0]) : (_Float16)0.f;
-            const _Float16 ma = sa * (_Float16)16.f, mb = sb * (_Float16)16.f;
-            const _Float16 na = sa * (_Float16)(ACT_UNSIGNED ? -16.f : -24.f), nb = sb * (_Float16)-24.f;
-            *(u32x2_t *)(base + STAGE_AS) = u32x2_t{as_u32(half2_t{ma, ma}), as_u32(half2_t{na, na})};
-            *(u32x2_t *)(base + STAGE_BS) = u32x2_t{as_u32(half2_t{mb, mb}), as_u32(half2_t{nb, nb})};
-        } else {
-            u32x4_t pa, pb;
+        u32x4_t pa, pb;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const _Float16 sa = (_Float16)ldexpf(e4m3_to_f32((ra >> (8 * j)) & 0x7Fu), c.shift);
-                pa[j] = as_u32(half2_t{sa, sa});
-                const uint32_t hb = c.col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
-                pb[j] = hb | (hb << 16);
-            }
-            *(u32x4_t *)(base + STAGE_AS) = pa;
-            *(u32x4_t *)(base + STAGE_BS) = pb;
+        for (int j = 0; j < 4; j++) {
+            const _Float16 sa = (_Float16)ldexpf(e4m3_to_f32((ra >> (8 * j)) & 0x7Fu), c.shift);
+            pa[j] = as_u32(half2_t{sa, sa});
+            const uint32_t hb = c.col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
+            pb[j] = hb | (hb << 16);
         }
+        *(u32x4_t *)(base + STAGE_AS) = pa;
+        *(u32x4_t *)(base + STAGE_BS) = pb;
     };
-
-    // conversion constants, pinned in registers (VOP3 cannot take literals; opaque values let the
-    // compiler form v_and_or_b32)
-    DequantConsts dc;
-    dc.magic = 0x3C003C00u;
-    dc.mask = 0x03C003C0u;
-    asm volatile("" : "+v"(dc.magic), "+s"(dc.mask));
 
     float16_t acc[4][4];
     int coltab_n0 = -1;  // first column of the tile whose column tables are in LDS (wave-uniform)
@@ -317,14 +249,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // safe against register copies and spills made before the data has arrived.
     auto load_scales_plain = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {
         const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
-        if (!FP4) {
-            ra = *(const uint16_t *)(c.as_base + (gc * as_stride + as_voff));
-            rb[0] = *(const uint16_t *)(c.bs_base + (gc * bs_stride + lane * BS_ELT));
-            rb[1] = 0;
-        } else {
-            ra = *(const uint32_t *)(c.as_base + (gc * as_stride + as_voff));
-            rb = *(const u32x2_t *)(c.bs_base + (gc * bs_stride + lane * BS_ELT));
-        }
+        ra = *(const uint32_t *)(c.as_base + (gc * as_stride + as_voff));
+        rb = *(const u32x2_t *)(c.bs_base + (gc * bs_stride + lane * BS_ELT));
     };
     auto issue_first_stages = [&](const TileCtx &c) {
         load_scales_plain(c, 0, s0a, s0b);
@@ -347,19 +273,15 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         for (int t = 0; t < 4; t++) {
             ar[t] = *(const u32x4_t *)(base + STAGE_A + (wm * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
             br[t] = *(const u32x4_t *)(base + STAGE_B + (wn * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
-            as[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 16 + (FP4 ? h * 8 : 0));
-            bs[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 16 + (FP4 ? h * 8 : 0));
+            as[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 16 + h * 8);
+            bs[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 16 + h * 8);
         }
     };
 #define SVDQ_CONVERT(AR, BR, AS, BS, I, A, B)                                                             \
     _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                       \
-        if (!FP4) {                                                                                       \
-            A[t] = dequant_word(AR[t][I], as_half2(AS[t][0]), as_half2(AS[t][1]), dc);                     \
-            B[t] = dequant_word(BR[t][I], as_half2(BS[t][0]), as_half2(BS[t][1]), dc);                     \
-        } else { /* word I of the lane's 32 codes lies in 16-group 2h + I/2 */                             \
-            A[t] = dequant_word_fp4(AR[t][I], as_half2(AS[t][(I) >> 1]));                                  \
-            B[t] = dequant_word_fp4(BR[t][I], as_half2(BS[t][(I) >> 1]));                                  \
-        }                                                                                                 \
+        /* word I of the lane's 32 codes lies in 16-group 2h + I/2 */                                     \
+        A[t] = dequant_word_fp4(AR[t][I], as_half2(AS[t][(I) >> 1]));                                      \
+        B[t] = dequant_word_fp4(BR[t][I], as_half2(BS[t][(I) >> 1]));                                      \
     }
 #define SVDQ_MFMA(A, B)                                                                                   \
     _Pragma("unroll") for (int mt = 0; mt < 4; mt++) _Pragma("unroll") for (int nt = 0; nt < 4; nt++)     \
@@ -390,7 +312,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 
   for (int batch0 = 0; batch0 < nseg; batch0 += MAX_BATCH) {
     const int nbatch = nseg - batch0 < MAX_BATCH ? nseg - batch0 : MAX_BATCH;
-    SVDQ_STAMP(0);
     {
     int tid_p = threadIdx.x;  // opaque copy: nothing derived from it is kept in registers beyond this block
     asm volatile("" : "+v"(tid_p));
@@ -398,57 +319,8 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // ---- largest activation scale of every row of the batch's tiles -> power-of-two shift that
     //      moves it into [2^10, 2^11)
     __syncthreads();  // the previous batch is done with the table
-    if (!FP4) {
-        // thread (oct, gs) takes the groups gs, gs + 8, ... of eight rows; the tiles of the batch go side
-        // by side through one loop so that their loads are in flight together (one memory latency per
-        // step, not one per tile and step)
-        for (int t = 0; t < nbatch; t++) rowshift[t * 256 + tid] = 0;
-        __syncthreads();
-        const int oct = tid & 31, gs = tid >> 5;
-        uint32_t mx[MAX_BATCH][8];
-        const uint16_t *src[MAX_BATCH];
-#pragma unroll
-        for (int t = 0; t < MAX_BATCH; t++) {
-            int m0, n0;
-            tile_coords(first_tile + batch0 + (t < nbatch ? t : 0), m0, n0);
-            src[t] = p.ascales + m0 + 8 * oct;
-#pragma unroll
-            for (int j = 0; j < 8; j++) mx[t][j] = 0;
-        }
-        for (int g = gs; g < kgroups; g += 24) {
-            // three steps of the group loop at once; slots beyond the batch read the batch's first tile
-            // again and steps beyond K the last group: no branches between the loads, all in flight together
-            u32x4_t v[3][MAX_BATCH];
-#pragma unroll
-            for (int u = 0; u < 3; u++) {
-                const int gu = g + 8 * u < kgroups ? g + 8 * u : kgroups - 1;
-#pragma unroll
-                for (int t = 0; t < MAX_BATCH; t++) v[u][t] = *(const u32x4_t *)(src[t] + (size_t)gu * p.M_pad);
-            }
-#pragma unroll
-            for (int u = 0; u < 3; u++)
-#pragma unroll
-                for (int t = 0; t < MAX_BATCH; t++) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        mx[t][2 * j] = max(mx[t][2 * j], v[u][t][j] & 0x7FFFu);
-                        mx[t][2 * j + 1] = max(mx[t][2 * j + 1], (v[u][t][j] >> 16) & 0x7FFFu);
-                    }
-                }
-        }
-#pragma unroll
-        for (int t = 0; t < MAX_BATCH; t++)
-            if (t < nbatch) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) atomicMax((uint32_t *)&rowshift[t * 256 + 8 * oct + j], mx[t][j]);
-            }
-        __syncthreads();
-        for (int t = 0; t < nbatch; t++) {
-            const int ex = rowshift[t * 256 + tid] >> 7;  // biased bf16 exponent of the row maximum
-            rowshift[t * 256 + tid] = ex == 0 ? 0 : NORM_TARGET_EXP - (ex - 127);
-        }
-    } else {
-        // NVFP4: four e4m3 scales per (row, 64-group) packed in one word; e4m3 patterns of
+    {
+        // four e4m3 scales per (row, 64-group) packed in one word; e4m3 patterns of
         // non-negative values order like unsigned bytes
         for (int t = 0; t < nbatch; t++) {
             int m0, n0;
@@ -466,7 +338,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     }
     }
     __syncthreads();
-    SVDQ_STAMP(1);
 
     TileCtx cur = make_ctx(batch0, 0, threadIdx.x, false, 0, 0, 0);
     issue_first_stages(cur);
@@ -475,11 +346,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     store_scales(cur, 1, s1a, s1b);
     store_scales(cur, 2, s2a, s2b);
     __syncthreads();
-    SVDQ_STAMP(2);
 
    for (int ti = 0; ti < nbatch; ti++) {
     const bool have_next = ti + 1 < nbatch;
-    SVDQ_STAMP_TILE(ti, 0);
     refresh_thread_coordinates();
     // A tile shared with the next workgroup (this one holds its first k-groups, the neighbour the rest):
     // the neighbour works on it first thing, so its partial sums are normally parked in the workspace by
@@ -528,22 +397,19 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // barrier that ends an iteration orders the reads of a stage before its refill)
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    // The compiler cannot see the waits issued from asm.  If it believes that one of its own loads (the
-    // next-layer epilogue has many) might still be in flight here, it protects the registers the loop's
-    // asm loads write with a full vmcnt(0) drain at the top of every iteration.  A wait through the
-    // builtin, which its bookkeeping understands, settles that before the loop.  In these variants the
-    // hand-over has waited for everything already; the plain INT4 variant, whose hand-over leaves output
-    // stores in flight on purpose, does not need it.
-    if (NEXT || FP4) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt unconstrained
+    // The compiler cannot see the waits issued from asm.  A wait through the builtin, which its
+    // bookkeeping understands, tells it that none of its own loads is in flight when the loop starts
+    // (the hand-over has waited for everything already).
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt unconstrained
     const int seg_len = cur.ge - cur.gb;  // even: segments begin and end on units of two k-groups
     for (int l = 0; l < seg_len; l += 2) {
-        issue_scales(cur, l + 3, sa_e, sb_e);
-        issue_scales(cur, l + 4, sa_o, sb_o);
         issue_codes(cur, l + 3);
         issue_codes(cur, l + 4);
+        issue_scales(cur, l + 3, sa_e, sb_e);
+        issue_scales(cur, l + 4, sa_o, sb_o);
         SVDQ_GROUP(l)
         SVDQ_GROUP(l + 1)
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(sa_e), "+v"(sb_e), "+v"(sa_o), "+v"(sb_o) :: "memory");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the copies (the compiler waits for the scale loads itself)
         store_scales(cur, l + 3, sa_e, sb_e);
         store_scales(cur, l + 4, sa_o, sb_o);
         __syncthreads();
@@ -555,7 +421,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                       "+a"(acc[1][2]), "+a"(acc[1][3]), "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]),
                       "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
     __syncthreads();
-    SVDQ_STAMP_TILE(ti, 1);
     // Thread coordinates for the epilogue, re-derived from an opaque copy of the thread index: nothing
     // computed from them can be hoisted above the main loop and occupy registers there.
     int tid_e = threadIdx.x;
@@ -614,8 +479,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         combine = last;
         if (last && tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
     }
-
-    SVDQ_STAMP_TILE(ti, 5);
     // ---- epilogue -----------------------------------------------------------------------------
     // The MFMAs were issued with the weight tile as the first operand, so a lane holds one output ROW
     // (r32 of the 32-row tile) and accumulator element e is COLUMN 8*(e/4) + 4*h + e%4 of the 32-column
@@ -643,13 +506,11 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // The projection is added to the accumulators BEFORE they are scaled.  The accumulators are in
     // normalised units (out = acc * rn[row] * cf[col] + bias), so the operands are divided by rn and cf
     // first; the matrix cores then update the accumulators in place and the operands are dead before the
-    // output pass starts.  INT4: rn and cf are powers of two (alpha is 1 and there are no per-channel
-    // scales), the division only changes exponents and the bf16 products are the same numbers.  NVFP4: cf
+    // output pass starts.  rn is a power of two (the division only changes exponents); cf
     // (column normalisation x alpha x wcscales) is an arbitrary number, so up / cf is passed as the sum of
     // two bf16 numbers (the rounded quotient and the rounded remainder: relative error 2^-17, below the
     // rounding noise of the main loop) in two matrix-core steps; wcscales must not be zero.
     const int nsteps = p.R_up / 16;
-    SVDQ_STAMP_TILE(ti, 6);
     if (run_epilogue && nsteps > 0) {
         {
             // two 16-rank steps per round; every request of a round is issued before any of its data is
@@ -670,13 +531,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                     const u32x4_t *bp = (const u32x4_t *)(p.lora_up + (size_t)(ok ? n : 0) * p.R_up + 8 * h);
                     rb[t][0] = bp[2 * s0];
                     rb[t][1] = bp[2 * s1];
-                    if (!FP4) {
-                        rcf[t] = ok ? __builtin_amdgcn_rcpf(p.colnorm[n]) : 0.f;  // of a power of two: exact
-                    } else {
-                        float cf = ok ? p.colnorm[n] * p.alpha : 1.f;
-                        if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
-                        rcf[t] = ok ? __fdiv_rn(1.0f, cf) : 0.f;
-                    }
+                    float cf = ok ? p.colnorm[n] * p.alpha : 1.f;
+                    if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
+                    rcf[t] = ok ? __fdiv_rn(1.0f, cf) : 0.f;
                     lsr[t] = ldexpf(1.0f, tile_shift[wm * 128 + t * 32 + r32]);
                 }
 #pragma unroll
@@ -699,7 +556,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                         for (int i = 0; i < 4; i++) {
                             const float q0 = bits_f32(bw[i] << 16) * rcf[t], q1 = bits_f32(bw[i] & 0xFFFF0000u) * rcf[t];
                             bw[i] = pack_bf16x2(q0, q1);
-                            if (FP4) br[i] = pack_bf16x2(q0 - bits_f32(bw[i] << 16), q1 - bits_f32(bw[i] & 0xFFFF0000u));
+                            br[i] = pack_bf16x2(q0 - bits_f32(bw[i] << 16), q1 - bits_f32(bw[i] & 0xFFFF0000u));
                         }
                         lb[t] = __builtin_bit_cast(bf16x8_t, bw);
                         lb_rem[t] = __builtin_bit_cast(bf16x8_t, br);
@@ -709,23 +566,19 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #pragma unroll
                         for (int nt = 0; nt < 4; nt++)
                             acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb[nt], la[mt], acc[mt][nt], 0, 0, 0);
-                    if (FP4) {
 #pragma unroll
-                        for (int mt = 0; mt < 4; mt++)
+                    for (int mt = 0; mt < 4; mt++)
 #pragma unroll
-                            for (int nt = 0; nt < 4; nt++)
-                                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb_rem[nt], la[mt], acc[mt][nt], 0, 0, 0);
-                    }
+                        for (int nt = 0; nt < 4; nt++)
+                            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb_rem[nt], la[mt], acc[mt][nt], 0, 0, 0);
                 }
             }
         }
     }
-    SVDQ_STAMP_TILE(ti, 7);
     // everything requested so far has arrived before the next tile's first stages are requested: a
     // wait on a later request would otherwise also wait for everything issued in between
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
-    SVDQ_STAMP_TILE(ti, 2);
     // first stages of the next tile: in flight while this tile's epilogue runs (the LDS stages are
     // free, the epilogue works in its own slab)
     if (have_next) issue_first_stages(nxt);
@@ -934,10 +787,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         float lo = bits_f32(v[j] << 16), hi = bits_f32(v[j] & 0xFFFF0000u);
-                        if (!FP4) {  // INT4 next layer: unsigned codes after a +0.171875 shift (launch_impl.cuh:286-294)
-                            lo = bf16_bits_to_f32(f32_to_bf16_bits(__fadd_rn(lo, 0.171875f)));
-                            hi = bf16_bits_to_f32(f32_to_bf16_bits(__fadd_rn(hi, 0.171875f)));
-                        }
                         y[8 * i + 2 * j] = smooth_quotient(lo, nrs[8 * i + 2 * j]);
                         y[8 * i + 2 * j + 1] = smooth_quotient(hi, nrs[8 * i + 2 * j + 1]);
                     }
@@ -945,16 +794,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 const int m = wrow0 + mt * 32 + rr;
                 const int gidx = (wcol0 + qc * 32) / 64;
                 u32x4_t words;
-                if (!FP4) {
-                    float sc;
-                    quantize_int4_half_group<true>(y, 1, words, sc);
-                    if ((qc & 1) == 0) ((uint16_t *)p.oscales)[(size_t)gidx * p.M_pad + m] = (uint16_t)f32_to_bf16_bits(sc);
-                } else {
-                    uint32_t sc[2];
-                    quantize_nvfp4_two_groups(y, words, sc);
-                    uint16_t *os = (uint16_t *)p.oscales;  // [N/64][M_pad][4]
-                    os[((size_t)gidx * p.M_pad + m) * 2 + (qc & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
-                }
+                uint32_t sc[2];
+                quantize_nvfp4_two_groups(y, words, sc);
+                uint16_t *os = (uint16_t *)p.oscales;  // [N/64][M_pad][4]
+                os[((size_t)gidx * p.M_pad + m) * 2 + (qc & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
                 *(u32x4_t *)(p.qout + ((size_t)(m / 32) * ngroups_out + gidx) * TILE_BYTES + (m % 32) * 32 + 16 * (qc & 1)) = words;
             }
         }
@@ -977,7 +820,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         slab_epilogue(std::integral_constant<int, 2>{}, std::true_type{});
         slab_epilogue(std::integral_constant<int, 3>{}, std::true_type{});
     }
-    SVDQ_STAMP_TILE(ti, 3);
     if (have_next) {
         // The code copies of the next tile must have landed.  s_waitcnt vmcnt(n) returns once at most n
         // requests are outstanding, so it proves that the copies are complete only if at least n
@@ -994,7 +836,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         store_scales(cur, 2, s2a, s2b);
     }
     __syncthreads();
-    SVDQ_STAMP_TILE(ti, 4);
    }  // tiles of the batch
   }    // batches
 #undef SVDQ_GROUP
@@ -1003,11 +844,18 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 }
 
 
-template <bool ACT_UNSIGNED, bool FP4, bool NEXT>
+template <bool NEXT>
 int launch_gemm_variant(const GemmParams &p, int nwg, hipStream_t stream) {
-    auto kern = gemm_w4a4_kernel<ACT_UNSIGNED, FP4, NEXT>;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+    auto kern = gemm_w4a4_kernel<NEXT>;
+    // the attribute is set once per device (racing first calls both set it, which is harmless)
+    static bool lds_reserved[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(SVDQ_ELAUNCH, "gemm: cannot identify the current device");
+    if (!lds_reserved[dev]) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+        lds_reserved[dev] = true;
+    }
     hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), LDS_BYTES, stream, p);
     return check_launch("gemm_w4a4");
 }

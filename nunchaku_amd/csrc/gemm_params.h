@@ -26,7 +26,6 @@ constexpr int NORM_TARGET_EXP = 10;
 
 
 struct GemmParams {
-    long long *stamps;  // debug builds only: per-workgroup phase timestamps
     const uint8_t *act;
     const uint16_t *ascales;
     const uint8_t *wgt;
@@ -59,5 +58,58 @@ struct GemmParams {
     float norm_eps;
 };
 
+
+// ---- INT4 GEMM on the fp6 matrix instruction (gemm6_kernel.h) -------------------------------------
+namespace g6 {
+constexpr int BM = 128, BN = 256;  // workgroup tile; 4 waves as 2 x 2, wave tile 64 x 128
+// One stage of the LDS ring holds one k-group of the workgroup's operands:
+//   4 activation fragments | 8 weight fragments | weight scales 256 x {4 s, 0, 0, 0} bf16 |
+//   activation scales 128 x bf16 | zeros (what the upper half-wave reads as its activation scale)
+constexpr int ST_A = 0, ST_W = 4 * FRAG_BYTES, ST_WS = ST_W + 8 * FRAG_BYTES, ST_AS = ST_WS + 256 * 8, ST_Z = ST_AS + 256;
+constexpr int STAGE_BYTES = ST_Z + 128;
+constexpr int STAGES = 3;
+constexpr int COPIES_PER_WAVE = 6;  // asynchronous copies every wave issues per k-group
+// epilogue (reuses the ring): per wave one 32-row slab of bf16, then the column tables
+constexpr int OUT_LD = 136;
+constexpr int SLAB_BYTES = 32 * OUT_LD * 2;
+constexpr int EP_TAB = 4 * SLAB_BYTES;     // float cf[256], bias[256]
+constexpr int EP_NORMW = EP_TAB + 2048;    // 4 waves x float [128]: RMS-norm weights of the wave's head
+constexpr int EP_FLAG = EP_NORMW + 2048;   // one word handed from thread 0 to the workgroup
+constexpr int EP_RED = EP_FLAG + 16;       // [2 row halves][2][64 lanes] x float4: the two column halves' low-rank sums meet here
+constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+static_assert(EP_RED + 2 * 2 * 64 * 16 <= LDS_BYTES, "the epilogue must fit the ring");
+
+struct Params {
+    const uint8_t *act;        // fragments [M_pad/128][K/64][4]
+    const uint16_t *ascales;   // bf16 [K/64][M_pad]
+    const uint8_t *wgt;        // fragments [ceil(N/256)][K/64][8]
+    const uint8_t *wscales;    // [ceil(N/256)][K/64][256] x {bf16 4 * scale, 0, 0, 0}
+    const uint16_t *bias;      // bf16 [N] or null
+    const uint16_t *wcscales;  // bf16 [N] or null
+    const float *lora_act;     // fp32 [M_pad][R_up]
+    const uint16_t *lora_up;   // bf16 [N][R_up]
+    uint16_t *out;             // bf16 [M_out][N_out] or null
+    // next-layer fusion
+    uint8_t *qout;                 // fragments [M_pad/128][N/64][4] of the next layer's activations
+    uint16_t *oscales;             // bf16 [N/64][M_pad]
+    const float *next_smooth_rcp;  // fp32 [N]
+    const bf16x8_t *next_down;     // native proj_down of the next layer
+    float *next_lora_out;          // fp32 [M_pad][R_down]
+    long long *next_lora_fix;      // [M_pad][R_down] fixed-point sums (zero between launches)
+    int *next_lora_cnt;            // [M_pad/128] arrival counters (zero between launches)
+    // tiles split along K: parked partial sums and one arrival counter per tile (zero between launches)
+    float *partials;
+    int *counters;
+    int kparts;
+    int M_pad, N, K, M_out, N_out, R_up, R_down;
+    float alpha;
+    float lora_scales[8];
+    int gelu, silu;
+    const uint16_t *norm_q, *norm_k;
+    const float *rotary;
+    int rot_rows, rope_cols;
+    float norm_eps;
+};
+}  // namespace g6
 
 }  // namespace svdq

@@ -30,7 +30,7 @@ namespace {
 
 struct QuantParams {
     const uint16_t *x;       // bf16 [M, K]
-    uint8_t *act;            // native tiles
+    uint8_t *act;            // INT4: E2M3 fragments [M_pad/128][K/64][4]; NVFP4: nibble tiles [M_pad/32][K/64][32][32 B]
     void *oscales;           // bf16 [K/64, M_pad] or fp8 [K/16, M_pad]
     const bf16x8_t *down;    // native proj_down
     float *lora_out;         // [M_pad, R]
@@ -149,22 +149,29 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
                     }
                 }
             }
-            const size_t tile = (size_t)(row / 32) * kgroups + (2 * c + (q >> 1));
-            uint8_t *dst = p.act + tile * TILE_BYTES + (row % 32) * 32 + 16 * (q & 1);
-            u32x4_t words;
             if (!FP4) {
+                // E2M3 fragments [M_pad/128][K/64][4]: this lane's 32 codes are one fragment slot
+                u32x4_t lo;
+                u32x2_t hi;
                 float s;
-                quantize_int4_half_group<false>(y, 16, words, s);
+                quantize_int4_half_group_e2m3<false>(y, 16, lo, hi, s);
                 // (both lanes of a group hold the same scale and store it: no branch)
                 ((uint16_t *)p.oscales)[(size_t)(2 * c + (q >> 1)) * p.M_pad + row] = (uint16_t)f32_to_bf16_bits(s);
+                uint8_t *frag = p.act + (((size_t)(row / ACT_BLOCK_ROWS) * kgroups + (2 * c + (q >> 1))) * 4 + (row % ACT_BLOCK_ROWS) / 32) * FRAG_BYTES;
+                const int slot = (row % 32) + 32 * (q & 1);
+                *(u32x4_t *)(frag + slot * 16) = lo;
+                *(u32x2_t *)(frag + 1024 + slot * 8) = hi;
             } else {
+                const size_t tile = (size_t)(row / 32) * kgroups + (2 * c + (q >> 1));
+                uint8_t *dst = p.act + tile * TILE_BYTES + (row % 32) * 32 + 16 * (q & 1);
+                u32x4_t words;
                 uint32_t sc[2];
                 quantize_nvfp4_two_groups(y, words, sc);
                 // NVFP4 scales: [K/64][M_pad][4] -- the four 16-groups of a 64-group side by side
                 uint16_t *os = (uint16_t *)p.oscales;
                 os[((size_t)(2 * c + (q >> 1)) * p.M_pad + row) * 2 + (q & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
+                *(u32x4_t *)dst = words;
             }
-            *(u32x4_t *)dst = words;
         }
 
         // ---- low-rank down projection on the raw activations (rank tiles beyond R repeat tile 0 into

@@ -13,10 +13,9 @@ namespace {
 // Reference storage (packer.py:210-239, loader gemm_base.cuh:278-294): u32 words
 // [N/128][K/64][j:8][lane:32][c:4]; word c of lane (g = lane/4, t = lane%4) in 16-row tile j holds
 // row 16j + g + 8*(c>=2), columns 32*(c odd) + 8t + [0..8), element e in bits [4e, 4e+4).
-// Native: [N/32][K/64][32 rows][8 words], word w of a row holds columns 8w + [0..8); INT4 words are
-// made offset-binary and rotated (svdq_common.h).
-__global__ void repack_qweight_kernel(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, int64_t N, int64_t K,
-                                      uint32_t xor_mask, int rot) {
+// Native form of NVFP4 weights: [N/32][K/64][32 rows][8 words], word w of a row holds columns
+// 8w + [0..8), plain nibbles.  (INT4 weights take the other kernel below.)
+__global__ void repack_qweight_kernel(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, int64_t N, int64_t K) {
     const int64_t total = N * K / 8;
     const int64_t kgroups = K / 64;
     for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
@@ -31,9 +30,48 @@ __global__ void repack_qweight_kernel(const uint32_t *__restrict__ src, uint32_t
         const int codd = w / 4, t = w % 4;
         const int lane = gl * 4 + t, c = chi * 2 + codd;
         const int64_t s = (((bn * kgroups + g) * 8 + j) * 32 + lane) * 4 + c;
-        const uint32_t word = src[s] ^ xor_mask;
-        dst[i] = rot ? rotl32(word, rot) : word;
+        dst[i] = src[s];
     }
+}
+
+// INT4 weights for the fp6 matrix instruction: E2M3 fragments [ceil(N/256)][K/64][8 fragments]
+// (svdq_common.h).  One thread per fragment slot = (row, half of the k-group): it gathers the four
+// reference words that hold the row's 32 codes of that half and writes the 192-bit string.
+__global__ void repack_qweight_e2m3_kernel(const uint32_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t N, int64_t K) {
+    const int64_t kgroups = K / 64;
+    const int64_t nblocks = (N + WGT_BLOCK_COLS - 1) / WGT_BLOCK_COLS;
+    const int64_t total = nblocks * kgroups * 8 * 64;
+    const int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int slot = (int)(i % 64);
+    const int frag = (int)((i / 64) % 8);
+    const int64_t g = (i / 512) % kgroups;
+    const int64_t nblk = i / (512 * kgroups);
+    const int64_t n = nblk * WGT_BLOCK_COLS + frag * 32 + slot % 32;
+    const int half = slot / 32;
+    unsigned long long bits[3] = {0, 0, 0};
+    if (n < N) {
+        const int64_t bn = n / 128;
+        const int nn = (int)(n % 128);
+        const int j16 = nn / 16, gl = nn % 8, chi = (nn % 16) / 8;
+        const int c = chi * 2 + half;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint32_t word = src[(((bn * kgroups + g) * 8 + j16) * 32 + (gl * 4 + t)) * 4 + c];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int nib = (word >> (4 * e)) & 0xF;
+                const unsigned long long pat = int4_code_to_e2m3(nib >= 8 ? nib - 16 : nib);
+                const int bit = 6 * (8 * t + e);
+                bits[bit / 64] |= pat << (bit % 64);
+                if (bit % 64 > 58) bits[bit / 64 + 1] |= pat >> (64 - bit % 64);
+            }
+        }
+    }
+    uint8_t *f = dst + ((nblk * kgroups + g) * 8 + frag) * FRAG_BYTES;
+    *(unsigned long long *)(f + slot * 16) = bits[0];
+    *(unsigned long long *)(f + slot * 16 + 8) = bits[1];
+    *(unsigned long long *)(f + 1024 + slot * 8) = bits[2];
 }
 
 // ---- 16-bit per-channel values in the reference "wscale" order ----------------------------------
@@ -46,28 +84,23 @@ __device__ inline int64_t wscale_src_index(int64_t g, int64_t n, int64_t G) {
     return ((bn * G + g) * 32 + (4 * a + c)) * 4 + (2 * b + d);
 }
 
-// exponent shift that puts the largest scale of a column into [2^10, 2^11): 16 * scale and 24 * scale
-// (the packed-fma constants of the GEMM) then stay below the fp16 maximum
-constexpr int NORM_TARGET_EXP = 10;
-
-__global__ void repack_wscales_kernel(const uint16_t *__restrict__ src, _Float16 *__restrict__ dst,
-                                      float *__restrict__ colnorm, int64_t N, int64_t G) {
-    const int64_t n = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
-    if (n >= N) return;
-    float amax = 0.f;
-    for (int64_t g = 0; g < G; g++) amax = fmaxf(amax, fabsf(bf16_bits_to_f32(src[wscale_src_index(g, n, G)])));
-    int e = 0;
-    if (amax > 0.f) {
-        int ex;
-        frexpf(amax, &ex);  // amax = m * 2^ex, m in [0.5, 1)  ->  amax in [2^(ex-1), 2^ex)
-        e = NORM_TARGET_EXP - (ex - 1);
-    }
-    for (int64_t g = 0; g < G; g++) {
-        const float s = bf16_bits_to_f32(src[wscale_src_index(g, n, G)]);
-        dst[g * N + n] = (_Float16)ldexpf(s, e);
-    }
-    colnorm[n] = ldexpf(1.0f, -e);
+// INT4 weight scales as the operand of the GEMM's factor MFMA: [ceil(N/256)][K/64][256 columns] x
+// {bf16(4 s), 0, 0, 0} (the 4 undoes the halving of both operands' codes; exact, a power of two).
+// Columns beyond N hold zero.
+__global__ void repack_wscales_kernel(const uint16_t *__restrict__ src, unsigned long long *__restrict__ dst, int64_t N, int64_t G) {
+    const int64_t nblocks = (N + WGT_BLOCK_COLS - 1) / WGT_BLOCK_COLS;
+    const int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+    if (i >= nblocks * G * WGT_BLOCK_COLS) return;
+    const int64_t n = (i / (G * WGT_BLOCK_COLS)) * WGT_BLOCK_COLS + i % WGT_BLOCK_COLS;
+    const int64_t g = (i / WGT_BLOCK_COLS) % G;
+    unsigned long long v = 0;
+    if (n < N) v = f32_to_bf16_bits(4.0f * bf16_bits_to_f32(src[wscale_src_index(g, n, G)]));
+    dst[i] = v;
 }
+
+// exponent shift that puts the largest NVFP4 scale of a column into [2^10, 2^11): the fp16 products
+// of the NVFP4 GEMM then stay below the fp16 maximum
+constexpr int NORM_TARGET_EXP = 10;
 
 // ---- NVFP4 micro scales --------------------------------------------------------------------------
 // Reference storage (packer.py:346-360, loader gemm_w4a4.cuh:75-83): bytes
@@ -186,19 +219,28 @@ int svdq_repack_qweight(const void *src, void *dst, int64_t N, int64_t K, int fp
     SVDQ_REQUIRE(src != dst, "repack_qweight: in-place repack is not supported");
     SVDQ_REQUIRE(N > 0 && K > 0 && N % 128 == 0 && K % 128 == 0, "repack_qweight: N (%lld) and K (%lld) must be multiples of 128",
                  (long long)N, (long long)K);
+    if (!fp4) {
+        const int64_t slots = ((N + WGT_BLOCK_COLS - 1) / WGT_BLOCK_COLS) * (K / 64) * 8 * 64;
+        SVDQ_REQUIRE((uintptr_t)dst % 16 == 0, "repack_qweight: dst must be 16-byte aligned");
+        hipLaunchKernelGGL(repack_qweight_e2m3_kernel, dim3(blocks_for(slots)), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
+                           (uint8_t *)dst, N, K);
+        return check_launch("repack_qweight");
+    }
     const int64_t total = N * K / 8;
     unsigned grid = blocks_for(total);
     if (grid > 65536u) grid = 65536u;
     hipLaunchKernelGGL(repack_qweight_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
-                       (uint32_t *)dst, N, K, fp4 ? 0u : 0x88888888u, fp4 ? 0 : INT4_WORD_ROT);
+                       (uint32_t *)dst, N, K);
     return check_launch("repack_qweight");
 }
 
-int svdq_repack_wscales(const void *src, void *dst_scales, void *dst_colnorm, int64_t N, int64_t K, void *stream) {
-    SVDQ_REQUIRE(src && dst_scales && dst_colnorm, "repack_wscales: null pointer");
+int svdq_repack_wscales(const void *src, void *dst_scales, int64_t N, int64_t K, void *stream) {
+    SVDQ_REQUIRE(src && dst_scales, "repack_wscales: null pointer");
     SVDQ_REQUIRE(N > 0 && K > 0 && N % 128 == 0 && K % 64 == 0, "repack_wscales: N %% 128 and K %% 64 must be 0");
-    hipLaunchKernelGGL(repack_wscales_kernel, dim3(blocks_for(N)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
-                       (_Float16 *)dst_scales, (float *)dst_colnorm, N, K / 64);
+    SVDQ_REQUIRE((uintptr_t)dst_scales % 16 == 0, "repack_wscales: dst must be 16-byte aligned");
+    const int64_t total = ((N + WGT_BLOCK_COLS - 1) / WGT_BLOCK_COLS) * (K / 64) * WGT_BLOCK_COLS;
+    hipLaunchKernelGGL(repack_wscales_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
+                       (unsigned long long *)dst_scales, N, K / 64);
     return check_launch("repack_wscales");
 }
 

@@ -76,19 +76,34 @@ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bf16x2_t));
 }
 
-// Native tile geometry of 4-bit operands (activations and weights alike):
-//   [rows/32][K/64][32 rows][8 words]; word w of a (row, 64-group) holds elements 8w .. 8w+7.
-//   NVFP4: element e of a word in bits [4e, 4e+4) (plain nibbles).
-//   INT4 : the same nibble word rotated left by 2 bits (INT4_WORD_ROT), signed codes offset-binary
-//          (code + 8).  The rotation puts elements 1 and 5 on bits [9:6] / [25:22], i.e. onto the top
-//          mantissa bits of an fp16 pair, and every other pair one shift or rotate away from there:
-//          OR-ing 0x3C00 gives the fp16 value 1 + u/16, and one packed fma with (16 s, -24 s) yields
-//          (u - 8) s exactly.
+// Native tile geometry of NVFP4 operands (activations and weights alike):
+//   [rows/32][K/64][32 rows][8 words]; word w of a (row, 64-group) holds elements 8w .. 8w+7, element e
+//   of a word in bits [4e, 4e+4) (plain E2M1 nibbles).
 constexpr int TILE_ROWS = 32;
 constexpr int GROUP_K = 64;
 constexpr int TILE_BYTES = TILE_ROWS * GROUP_K / 2;  // 1024
-constexpr int INT4_WORD_ROT = 2;
 
 __host__ __device__ inline uint32_t rotl32(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
+
+// INT4 operands of the GEMM (activations and weights alike) are stored as E2M3 (fp6) patterns of
+// code / 2, which is exact for every code in [-8, 15]: the fp6 matrix instruction then multiplies the
+// bare codes at twice the INT8 rate and returns fp32.  A "fragment" is one operand of
+// v_mfma_f32_32x32x64_f8f6f4: 32 rows x 64 codes (one k-group) = 1536 bytes.  Slot s = row + 32 * half
+// (half = which 32 of the 64 codes) owns the 192-bit string with code j of its half in bits
+// [6 j, 6 j + 6); the first 16 bytes of the string are stored at 16 s, the last 8 at 1024 + 8 s, so that
+// a wave fetches a fragment with one 16-byte and one 8-byte LDS read per lane, both conflict-free.
+// Fragments are grouped per workgroup tile: activations [M_pad/128][K/64][4 fragments], weights
+// [ceil(N/256)][K/64][8 fragments] (columns beyond N hold zero codes): a workgroup's operands of one
+// k-group are one contiguous run of 6 KB and one of 12 KB.
+constexpr int FRAG_BYTES = 1536;
+constexpr int ACT_BLOCK_ROWS = 128, WGT_BLOCK_COLS = 256;
+
+// E2M3 pattern of code / 2 for an integer code in [-15, 15] (bias 1, subnormals, no inf / nan):
+// magnitudes 0..3 are (x << 2), 4..7 are 8 + 2 x, 8..15 are 16 + x; the sign is bit 5.
+__host__ __device__ inline uint32_t int4_code_to_e2m3(int code) {
+    const uint32_t x = code < 0 ? -code : code;
+    const uint32_t m = x < 4 ? x << 2 : (x < 8 ? 8 + 2 * x : 16 + x);
+    return m | (code < 0 ? 32u : 0u);
+}
 
 }  // namespace svdq

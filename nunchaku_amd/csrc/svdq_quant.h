@@ -22,20 +22,6 @@ __device__ inline float smooth_quotient(float x, float rcp) {
     return bf16_bits_to_f32(f32_to_bf16_bits(__fmul_rn(x, rcp)));
 }
 
-// 8 clamped-and-rounded codes (already offset so that they are in [0, 15]) -> one word.  Every input is
-// RNE_MAGIC + u, bit pattern 0x4B400000 | u: bits [21:4] are zero, so four of them chain into 16 clean
-// low bits with shift-and-or alone (the constant's bits stay at or above bit 22), and one byte
-// permute joins the two halves: 7 instructions per word.
-__device__ inline uint32_t pack8(const float (&v)[8]) {
-    uint32_t lo = f32_bits(v[3]), hi = f32_bits(v[7]);
-#pragma unroll
-    for (int j = 2; j >= 0; j--) {
-        lo = (lo << 4) | f32_bits(v[j]);
-        hi = (hi << 4) | f32_bits(v[4 + j]);
-    }
-    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes 0, 1 of lo below bytes 0, 1 of hi
-}
-
 // fp32 (finite, >= 0, <= 448) -> e4m3 bit pattern, round to nearest even
 __device__ inline uint32_t f32_to_e4m3(float s) {
     if (s < 0.0009765625f) return 0;  // below half of the smallest subnormal (2^-10) rounds to 0
@@ -79,31 +65,31 @@ __device__ inline uint32_t pack8_e2m1(const float (&t)[8]) {
 }
 
 
-// One lane holds 32 consecutive elements of a row = half of a 64-group; the other half lives in the
-// lane `partner_xor` away.  Produces the 16 bytes of codes of this half and the group scale.
-// Signed codes are emitted offset-binary (code + 8), unsigned ones as they are; words are in the
-// rotated INT4 word format of svdq_common.h.
+// INT4: one lane holds 32 consecutive elements of a row = half of a 64-group; the other half lives in
+// the lane `partner_xor` away.  The 32 codes of the lane leave as the E2M3
+// patterns of code / 2, 6 bits each, code j in bits [6 j, 6 j + 6) of a 192-bit string (`lo` = bits
+// [0, 128), `hi` = the rest).  The hardware conversion takes the even and the odd elements as two
+// sources and interleaves them; dividing the already rounded and clamped integer by its scale operand
+// (2) is exact.
 template <bool UNSIGNED>
-__device__ inline void quantize_int4_half_group(const float (&y)[32], int partner_xor, u32x4_t &words, float &scale) {
+__device__ inline void quantize_int4_half_group_e2m3(const float (&y)[32], int partner_xor, u32x4_t &lo, u32x2_t &hi, float &scale) {
+    typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
     float amax = 0.f;
 #pragma unroll
     for (int e = 0; e < 32; e++) amax = fmaxf(amax, fabsf(y[e]));
     amax = fmaxf(amax, __shfl_xor(amax, partner_xor));
     const float s = __fmul_rn(amax, UNSIGNED ? RECIP_15 : RECIP_7);
     const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
-    const float lo = UNSIGNED ? 0.0f : -8.0f, hi = UNSIGNED ? 15.0f : 7.0f;
-    const float magic = UNSIGNED ? RNE_MAGIC : RNE_MAGIC + 8.0f;
+    const float cl = UNSIGNED ? 0.0f : -8.0f, ch = UNSIGNED ? 15.0f : 7.0f;
+    float16_t ev, od;
 #pragma unroll
-    for (int wi = 0; wi < 4; wi++) {
-        float v[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            float t = __fmul_rn(y[8 * wi + j], rcp);
-            t = fminf(fmaxf(t, lo), hi);
-            v[j] = __fadd_rn(t, magic);  // the rounded code sits in the low nibble of the bit pattern
-        }
-        words[wi] = rotl32(pack8(v), INT4_WORD_ROT);
+    for (int e = 0; e < 16; e++) {
+        ev[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e], rcp), cl, ch));
+        od[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e + 1], rcp), cl, ch));
     }
+    const u32x6_t w = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, 2.0f);
+    lo = u32x4_t{w[0], w[1], w[2], w[3]};
+    hi = u32x2_t{w[4], w[5]};
     scale = s;
 }
 

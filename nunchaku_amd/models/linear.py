@@ -67,6 +67,7 @@ class SVDQW4A4Linear(nn.Module):
 
         self.act_unsigned = act_unsigned
         self._native: dict[str, torch.Tensor | None] | None = None
+        self._native_stamp: tuple | None = None
         self._alpha: float | None = None
 
     @classmethod
@@ -83,17 +84,40 @@ class SVDQW4A4Linear(nn.Module):
 
     # ---- load-time repack -------------------------------------------------------------------
     def _load_from_state_dict(self, *args, **kwargs):
-        self._native = None  # new checkpoint tensors: convert again on next use
-        self._alpha = None
+        self.invalidate_native()  # new checkpoint tensors: convert again on next use
         return super()._load_from_state_dict(*args, **kwargs)
 
     def _apply(self, fn, *args, **kwargs):
-        self._native = None
+        self.invalidate_native()
         return super()._apply(fn, *args, **kwargs)
 
+    _NATIVE_SOURCES = ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias", "wcscales", "wtscale")
+
+    def _stamp(self) -> tuple:
+        """Identity and in-place modification counter of every parameter the native tensors come from."""
+        out = []
+        for name in self._NATIVE_SOURCES:
+            t = getattr(self, name, None)
+            out.append(None if t is None else (t.data_ptr(), packing.tensor_version(t)))
+        return tuple(out)
+
+    def invalidate_native(self) -> None:
+        """Forget the converted tensors (and the cached ``alpha``): the next use converts again.  Needed
+        only after writes that leave no trace on the parameters (``param.data.copy_(...)``, or any write
+        to inference-mode tensors); in-place operations on the parameters themselves, ``load_state_dict``
+        and ``.to()`` are noticed without it."""
+        self._native = None
+        self._native_stamp = None
+        self._alpha = None
+
     def native_tensors(self) -> dict[str, torch.Tensor | None]:
-        """The layer's tensors in the layouts the kernels read, converted on first use."""
+        """The layer's tensors in the layouts the kernels read, converted on first use and again after
+        a parameter has been replaced or modified in place (a low-rank swap, for example)."""
+        stamp = self._stamp()
+        if self._native is not None and stamp != self._native_stamp:
+            self.invalidate_native()
         if self._native is None:
+            self._native_stamp = stamp
             fp4 = self.precision == "nvfp4"
             self._native = {
                 "qweight": packing.repack_qweight(self.qweight.data, fp4),
@@ -110,6 +134,7 @@ class SVDQW4A4Linear(nn.Module):
     def alpha(self) -> float:
         """Per-tensor weight scale as a host float, read once (the reference hands the parameter to a
         ``float`` argument on every call, nunchaku/models/linear.py:128, which synchronises)."""
+        self.native_tensors()  # (drops a stale value when wtscale was modified)
         if self._alpha is None:
             self._alpha = 1.0 if self.wtscale is None else float(self.wtscale.detach().float().cpu().item())
         return self._alpha

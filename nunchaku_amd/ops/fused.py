@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from ..packing import act_nbytes_per_row
 from ..utils import ceil_divide
 from .gemm import svdq_gemm_w4a4
 
@@ -16,7 +17,7 @@ def fused_gelu_mlp(x: torch.Tensor, fc1, fc2, pad_size: int = 256) -> torch.Tens
     quantized_x, ascales, lora_act = fc1.quantize(x)
 
     batch_size_pad = ceil_divide(batch_size * seq_len, pad_size) * pad_size
-    qout_act = torch.empty(batch_size_pad, fc1.out_features // 2, dtype=torch.uint8, device=x.device)
+    qout_act = torch.empty(batch_size_pad, act_nbytes_per_row(fc1.out_features, fc2.precision == "nvfp4"), dtype=torch.uint8, device=x.device)
     if fc2.precision == "nvfp4":
         qout_ascales = torch.empty(fc1.out_features // 16, batch_size_pad, dtype=torch.float8_e4m3fn, device=x.device)
     else:

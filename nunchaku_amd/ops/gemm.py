@@ -14,6 +14,24 @@ from .. import packing
 
 _NOT_BUILT = ("poolout", "out_vk", "out_linearattn", "out_q", "out_k", "out_v")
 NORM_EPS = 1e-6  # gemm_w4a4_launch_impl.cuh:374
+# Tuning / testing knob handed to the C ABI as ``k_split``: None lets the library decide, n > 0 splits
+# every output tile along K into n parts (1: never split).  No counterpart in the reference.
+K_SPLIT: int | None = None
+
+
+def _expect(name: str, t: torch.Tensor | None, shape: tuple, dtype: torch.dtype | None, dev: torch.device) -> None:
+    """The kernel reads and writes every row of these buffers: a wrong shape is an out-of-bounds access
+    on the device, so it is refused here (the reference asserts the same shapes in
+    gemm_w4a4_launch_impl.cuh:60-170)."""
+    if t is None:
+        return
+    nv.require_gpu(t, name)
+    if t.device != dev:
+        raise ValueError(f"svdq_gemm_w4a4: `{name}` is on {t.device}, the activations on {dev}")
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"svdq_gemm_w4a4: `{name}` has shape {tuple(t.shape)}, expected {tuple(shape)}")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"svdq_gemm_w4a4: `{name}` has dtype {t.dtype}, expected {dtype}")
 
 
 def svdq_gemm_w4a4(
@@ -49,7 +67,8 @@ def svdq_gemm_w4a4(
 ) -> None:
     """W4A4 GEMM with fused bias, low-rank up projection, optional GELU and next-layer quantization.
 
-    act      u8 [M_pad, K/2] and ``ascales`` [K/G, M_pad], as returned by the quantize operator;
+    act      u8 [M_pad, 3K/4] (INT4; [M_pad, K/2] for NVFP4) and ``ascales`` [K/G, M_pad], as returned by the
+    quantize operator (the byte layout is private to the two operators);
     wgt / wscales / lora_up / bias / wcscales / smooth_factor / lora_down: the layer's tensors, in
     the reference checkpoint layout (repacked once and cached) or already native (``packing``);
     out      bf16 [M, N] (M <= M_pad);  qout / oscales / lora_act_out: inputs of the next layer, in
@@ -91,9 +110,41 @@ def svdq_gemm_w4a4(
     if isinstance(alpha, torch.Tensor):  # the reference passes the wtscale parameter here (linear.py:128)
         alpha = float(alpha.item()) if alpha.numel() == 1 else 1.0
 
-    M_pad, K = act.shape[0], act.shape[1] * 2
-    N = wgt.shape[0]
+    if act.dim() != 2 or act.dtype != torch.uint8:
+        raise ValueError("svdq_gemm_w4a4: `act` must be the uint8 [M_pad, bytes] tensor written by the quantize operator")
+    M_pad = act.shape[0]
     dev = act.device
+    if packing.is_native(wgt, "qweight"):
+        N, K = wgt.logical_shape
+    else:
+        N, K = wgt.shape[0], wgt.shape[1] * 2
+    if M_pad % 256 != 0 or act.shape[1] != packing.act_nbytes_per_row(K, fp4):
+        raise ValueError(
+            f"svdq_gemm_w4a4: `act` has shape {tuple(act.shape)}; a layer with K={K} takes [M_pad, {packing.act_nbytes_per_row(K, fp4)}] "
+            "with M_pad a multiple of 256 (the activation layout is private to the two operators)")
+    G = 16 if fp4 else 64
+    sdt = torch.float8_e4m3fn if fp4 else torch.bfloat16
+    _expect("ascales", ascales, (K // G, M_pad), sdt, dev)
+    if not packing.is_native(wscales, "wscales"):
+        _expect("wscales", wscales, (K // G, N), sdt, dev)
+    for name, t in (("bias", bias), ("wcscales", wcscales)):
+        _expect(name, t, (N,), torch.bfloat16, dev)
+    if lora_up is not None:
+        _expect("lora_up", lora_up, (N, rank_up), torch.bfloat16, dev)
+        _expect("lora_act_in", lora_act_in, (M_pad, rank_up), torch.float32, dev)
+    if out is not None:
+        nv.require_gpu(out, "out")
+        if out.dtype != torch.bfloat16:
+            raise NotImplementedError("only bf16 outputs are supported")
+        if out.device != dev:
+            raise ValueError("svdq_gemm_w4a4: `out` is on another device")
+    if qout is not None:
+        _expect("qout", qout, (M_pad, packing.act_nbytes_per_row(N, fp4)), torch.uint8, dev)
+        _expect("oscales", oscales, (N // G, M_pad), sdt, dev)
+        _expect("smooth_factor", smooth_factor, (N,), None, dev)
+    if lora_down is not None:
+        _expect("lora_down", lora_down, (N, lora_down.shape[1]), torch.bfloat16, dev)
+        _expect("lora_act_out", lora_act_out, (M_pad, lora_down.shape[1]), torch.float32, dev)
     wgt_n = packing.native(wgt, "qweight", fp4)
     wsc_n = packing.native(wscales, "wscales", fp4)
     bias_n = packing.native(bias, "vector")
@@ -101,11 +152,6 @@ def svdq_gemm_w4a4(
     up_n = packing.native(lora_up, "lora_up")
     nsm_n = packing.native(smooth_factor, "smooth_rcp") if qout is not None else None
     ndown_n = packing.native(lora_down, "lora_down")
-    for name, t in (("out", out), ("qout", qout), ("oscales", oscales), ("lora_act_in", lora_act_in), ("lora_act_out", lora_act_out)):
-        if t is not None:
-            nv.require_gpu(t, name)
-    if out is not None and out.dtype != torch.bfloat16:
-        raise NotImplementedError("only bf16 outputs are supported")
 
     rot_n = None
     if rotary_emb is not None:
@@ -123,7 +169,7 @@ def svdq_gemm_w4a4(
     N_out = 0 if out is None else out.shape[-1]
     args = nv.GemmArgs(
         act=act.data_ptr(), ascales=ascales.data_ptr(), wgt=wgt_n.data_ptr(), wscales=wsc_n.data_ptr(),
-        colnorm=wsc_n.colnorm.data_ptr(), bias=nv.ptr(bias_n), wcscales=nv.ptr(wcs_n),
+        colnorm=nv.ptr(wsc_n.colnorm), bias=nv.ptr(bias_n), wcscales=nv.ptr(wcs_n),
         lora_act_in=nv.ptr(lora_act_in), lora_up=nv.ptr(up_n), lora_scales=sc, out=nv.ptr(out),
         qout=nv.ptr(qout), oscales=nv.ptr(oscales), next_smooth_rcp=nv.ptr(nsm_n),
         next_lora_down=nv.ptr(ndown_n), next_lora_act_out=nv.ptr(lora_act_out),
@@ -131,9 +177,10 @@ def svdq_gemm_w4a4(
         R_down=0 if lora_down is None else lora_down.shape[1],
         alpha=float(alpha), act_unsigned=int(act_unsigned), fuse_silu=int(fuse_silu), fp4=int(fp4),
         norm_q=nv.ptr(norm_q), norm_k=nv.ptr(norm_k), rotary_emb=nv.ptr(rot_n),
-        rot_rows=0 if rot_n is None else rot_n.shape[0], norm_eps=NORM_EPS,
+        rot_rows=0 if rot_n is None else rot_n.shape[0], norm_eps=NORM_EPS, k_split=int(K_SPLIT or 0),
     )
-    nv.check(nv.lib().svdq_gemm_w4a4(ctypes.byref(args), nv.stream_ptr(dev)))
+    with torch.cuda.device(dev):  # the library launches on the current device
+        nv.check(nv.lib().svdq_gemm_w4a4(ctypes.byref(args), nv.stream_ptr(dev)))
 
 
 svdq_gemm_w4a4_cuda = svdq_gemm_w4a4

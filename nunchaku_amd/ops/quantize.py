@@ -28,9 +28,11 @@ def svdq_quantize_w4a4_act_fuse_lora(
 
     input  bf16 [M, K];  lora_down  proj_down [K, R];  smooth  smooth_factor [K] (both either in the
     reference checkpoint layout, repacked once and cached, or already native, see ``packing``).
-    Returns ``(output u8 [M_pad, K/2], oscales [K/G, M_pad], lora_act_out fp32 [M_pad, R])`` where
-    M_pad rounds M up to ``pad_size`` (256).  ``output`` uses the kernels' private tile layout
-    (``packing.act_to_logical`` gives one code per element).
+    Returns ``(output u8 [M_pad, 3K/4], oscales [K/G, M_pad], lora_act_out fp32 [M_pad, R])`` where
+    M_pad rounds M up to ``pad_size`` (256).  ``output`` is private to this operator and the GEMM: INT4
+    codes travel as 6-bit E2M3 patterns, the matrix-core operand format (the reference's tensor is
+    [M_pad, K/2], also in a private order); NVFP4 keeps [M_pad, K/2].  ``packing.act_to_logical`` gives
+    one code per element.
     """
     if input.dim() != 2:
         raise ValueError("input must be [M, K]")
@@ -46,7 +48,7 @@ def svdq_quantize_w4a4_act_fuse_lora(
     batch_size_pad = ceil_divide(batch_size, pad_size) * pad_size
     dev = input.device
     if output is None:
-        output = torch.empty(batch_size_pad, channels // 2, dtype=torch.uint8, device=dev)
+        output = torch.empty(batch_size_pad, packing.act_nbytes_per_row(channels, fp4), dtype=torch.uint8, device=dev)
     if oscales is None:
         if fp4:
             assert channels % 16 == 0
@@ -58,8 +60,19 @@ def svdq_quantize_w4a4_act_fuse_lora(
         lora_act_out = torch.empty(batch_size_pad, rank, dtype=torch.float32, device=dev)
     for name, t in (("output", output), ("oscales", oscales), ("lora_act_out", lora_act_out)):
         nv.require_gpu(t, name)
-    if tuple(output.shape) != (batch_size_pad, channels // 2) or tuple(lora_act_out.shape) != (batch_size_pad, rank):
-        raise ValueError("output / lora_act_out have the wrong shape")
+    if tuple(output.shape) != (batch_size_pad, packing.act_nbytes_per_row(channels, fp4)) or output.dtype != torch.uint8:
+        raise ValueError(
+            f"output must be uint8 [{batch_size_pad}, {packing.act_nbytes_per_row(channels, fp4)}] (6 bits per INT4 element: the "
+            "activation layout is private to the two operators), got " + str(tuple(output.shape)))
+    if tuple(lora_act_out.shape) != (batch_size_pad, rank) or lora_act_out.dtype != torch.float32:
+        raise ValueError(f"lora_act_out must be float32 [{batch_size_pad}, {rank}]")
+    G = 16 if fp4 else 64
+    if tuple(oscales.shape) != (channels // G, batch_size_pad) or oscales.dtype != (torch.float8_e4m3fn if fp4 else torch.bfloat16):
+        raise ValueError(f"oscales must be [{channels // G}, {batch_size_pad}] of {'float8_e4m3fn' if fp4 else 'bfloat16'}")
+    if tuple(lora_down.shape) != (channels, rank):
+        raise ValueError(f"lora_down must be [{channels}, R], got {tuple(lora_down.shape)}")
+    if smooth is not None and smooth.numel() != channels:
+        raise ValueError(f"smooth must have {channels} elements")
 
     down = packing.native(lora_down, "lora_down")
     rcp = packing.native(smooth, "smooth_rcp")
@@ -68,7 +81,8 @@ def svdq_quantize_w4a4_act_fuse_lora(
         lora_down=nv.ptr(down) if rank else None, lora_act_out=lora_act_out.data_ptr() if rank else None, smooth_rcp=nv.ptr(rcp),
         M=batch_size, M_pad=batch_size_pad, K=channels, R=rank, fp4=int(fp4), fuse_glu=int(fuse_glu),
     )
-    nv.check(nv.lib().svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(args), nv.stream_ptr(dev)))
+    with torch.cuda.device(dev):  # the library launches on the current device
+        nv.check(nv.lib().svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(args), nv.stream_ptr(dev)))
     return output, oscales, lora_act_out
 
 

@@ -29,27 +29,42 @@ def is_native(t: torch.Tensor | None, kind: str) -> bool:
     return t is not None and getattr(t, NATIVE_ATTR, None) == kind
 
 
+FRAG_BYTES = 1536  # one fp6 MFMA operand: 32 rows x 64 codes x 6 bits (csrc/svdq_common.h)
+ACT_BLOCK_ROWS, WGT_BLOCK_COLS = 128, 256
+
+
 def repack_qweight(qweight: torch.Tensor, fp4: bool = False) -> torch.Tensor:
-    """int8 [N, K/2] reference order -> int8 [N, K/2] native tiles (offset-binary INT4 codes)."""
+    """int8 [N, K/2] reference order -> native weights.  INT4: E2M3 fragments
+    ``[ceil(N/256)][K/64][8]`` as int8 ``[ceil(N/256) * 256, 3K/4]`` (``.logical_shape`` = (N, K));
+    NVFP4: int8 [N, K/2] nibble tiles."""
     nv.require_gpu(qweight, "qweight")
     N, K2 = qweight.shape
-    out = torch.empty_like(qweight)
-    nv.check(nv.lib().svdq_repack_qweight(qweight.data_ptr(), out.data_ptr(), N, K2 * 2, int(fp4), nv.stream_ptr(qweight.device)))
-    return _tag(out, "qweight")
+    K = K2 * 2
+    if fp4:
+        out = torch.empty_like(qweight)
+    else:
+        n_pad = (N + WGT_BLOCK_COLS - 1) // WGT_BLOCK_COLS * WGT_BLOCK_COLS
+        out = torch.empty(n_pad, K * 3 // 4, dtype=torch.int8, device=qweight.device)
+    nv.check(nv.lib().svdq_repack_qweight(qweight.data_ptr(), out.data_ptr(), N, K, int(fp4), nv.stream_ptr(qweight.device)))
+    return _tag(out, "qweight", logical_shape=(N, K))
 
 
 def repack_wscales(wscales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
-    """bf16 [K/64, N] (or fp8 [K/16, N]) reference order -> fp16 column-normalised scales with the
-    same element count (INT4: ``[K/64][N]``; NVFP4: ``[K/64][N][4]`` viewed as ``[K/16, N]``); the
-    fp32 per-column factor that undoes the normalisation rides along as ``.colnorm``."""
+    """Reference-order group scales -> native.  INT4 (bf16 [K/64, N]): the factor operand
+    ``[ceil(N/256)][K/64][256] x {bf16(4 s), 0, 0, 0}`` as int64 ``[ceil(N/256), K/64, 256]``.
+    NVFP4 (fp8 [K/16, N]): fp16 column-normalised ``[K/64][N][4]`` viewed as ``[K/16, N]``, with the
+    fp32 per-column factor that undoes the normalisation as ``.colnorm``."""
     nv.require_gpu(wscales, "wscales")
     G, N = wscales.shape
-    out = torch.empty(G, N, dtype=torch.float16, device=wscales.device)
-    colnorm = torch.empty(N, dtype=torch.float32, device=wscales.device)
-    fn = nv.lib().svdq_repack_wmscales if fp4 else nv.lib().svdq_repack_wscales
-    K = G * (16 if fp4 else 64)
-    nv.check(fn(wscales.data_ptr(), out.data_ptr(), colnorm.data_ptr(), N, K, nv.stream_ptr(wscales.device)))
-    return _tag(out, "wscales", colnorm=colnorm)
+    if fp4:
+        out = torch.empty(G, N, dtype=torch.float16, device=wscales.device)
+        colnorm = torch.empty(N, dtype=torch.float32, device=wscales.device)
+        nv.check(nv.lib().svdq_repack_wmscales(wscales.data_ptr(), out.data_ptr(), colnorm.data_ptr(), N, G * 16, nv.stream_ptr(wscales.device)))
+        return _tag(out, "wscales", colnorm=colnorm)
+    nblocks = (N + WGT_BLOCK_COLS - 1) // WGT_BLOCK_COLS
+    out = torch.empty(nblocks, G, WGT_BLOCK_COLS, dtype=torch.int64, device=wscales.device)
+    nv.check(nv.lib().svdq_repack_wscales(wscales.data_ptr(), out.data_ptr(), N, G * 64, nv.stream_ptr(wscales.device)))
+    return _tag(out, "wscales", colnorm=None)
 
 
 def repack_vector(vec: torch.Tensor) -> torch.Tensor:
@@ -119,12 +134,27 @@ _REPACKERS = {
 _cache: dict[tuple, tuple[weakref.ref, torch.Tensor]] = {}
 
 
+def tensor_version(t: torch.Tensor) -> int | None:
+    """The in-place modification counter of ``t``, or None for tensors that keep none (those created
+    under ``torch.inference_mode()``)."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
 def native(t: torch.Tensor | None, kind: str, fp4: bool = False) -> torch.Tensor | None:
     """Return the native form of ``t``: ``t`` itself when it already is native, else a cached repack
-    of the reference-format tensor (redone when the source is modified or replaced)."""
+    of the reference-format tensor.  The cache notices in-place operations on the tensor and its
+    replacement (version counter, identity); a tensor without a version counter (inference mode) is
+    repacked on every call, and writes through ``t.data`` are invisible to it: pass native tensors
+    (``repack_*``) where that matters."""
     if t is None or is_native(t, kind):
         return t
-    key = (t.data_ptr(), t._version, tuple(t.shape), t.dtype, kind, fp4)
+    version = tensor_version(t)
+    if version is None:
+        return _REPACKERS[kind](t, fp4) if kind in ("qweight", "wscales") else _REPACKERS[kind](t)
+    key = (t.data_ptr(), version, tuple(t.shape), t.dtype, kind, fp4)
     hit = _cache.get(key)
     if hit is not None and hit[0]() is t:
         return hit[1]
@@ -140,36 +170,84 @@ def native(t: torch.Tensor | None, kind: str, fp4: bool = False) -> torch.Tensor
 # ---------------------------------------------------------------------------------------------
 
 
-INT4_WORD_ROT = 2  # INT4 code words are stored rotated left by this many bits (csrc/svdq_common.h)
+def act_nbytes_per_row(K: int, fp4: bool = False) -> int:
+    """Bytes of quantized activations per row: 4 bits per element for NVFP4, 6 (E2M3) for INT4."""
+    return K // 2 if fp4 else K * 3 // 4
+
+
+# E2M3 pattern of code / 2 for code in [-8, 15] (csrc/svdq_common.h, int4_code_to_e2m3), and its inverse
+def _e2m3_of_code(code: int) -> int:
+    x = abs(code)
+    m = x << 2 if x < 4 else (8 + 2 * x if x < 8 else 16 + x)
+    return m | (32 if code < 0 else 0)
+
+
+_E2M3_TO_CODE = torch.full((64,), 127, dtype=torch.int8)
+for _c in range(-15, 16):
+    _E2M3_TO_CODE[_e2m3_of_code(_c)] = _c
+_E2M3_TO_CODE[32] = 0  # minus zero: what the hardware conversion makes of a value that rounds to -0.0
+_CODE_TO_E2M3 = torch.tensor([_e2m3_of_code(c) for c in range(-16, 16)], dtype=torch.uint8)  # index code + 16
 
 
 def act_to_logical(act: torch.Tensor, K: int, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:
-    """Native activation tiles u8 [M_pad, K/2] ([M_pad/32][K/64][32 rows][8 words]) -> one code per
-    element, int8 [M_pad, K] in row/column order.  INT4 words are stored rotated left by 2 bits and
-    signed codes offset-binary (code + 8); NVFP4 words are plain nibbles."""
+    """Quantized activations in the kernels' private layout -> one code per element, int8 [M_pad, K] in
+    row/column order.  INT4: E2M3 fragments ``[M_pad/128][K/64][4]`` (u8 [M_pad, 3K/4]); NVFP4: nibble
+    tiles ``[M_pad/32][K/64][32 rows][8 words]`` (u8 [M_pad, K/2])."""
     M_pad = act.shape[0]
-    w = act.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
-    if not fp4:
-        w = ((w >> INT4_WORD_ROT) | (w << (32 - INT4_WORD_ROT))) & 0xFFFFFFFF
-    nib = torch.stack([(w >> (4 * e)) & 0xF for e in range(8)], dim=-1)  # [M_pad, K/8, 8] in tile order
-    codes = nib.reshape(M_pad // 32, K // 64, 32, 64).permute(0, 2, 1, 3).reshape(M_pad, K)
-    if not fp4 and not unsigned:
-        codes = codes - 8
-    return codes.to(torch.int8)
+    if fp4:
+        w = act.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+        nib = torch.stack([(w >> (4 * e)) & 0xF for e in range(8)], dim=-1)  # [M_pad, K/8, 8] in tile order
+        return nib.reshape(M_pad // 32, K // 64, 32, 64).permute(0, 2, 1, 3).reshape(M_pad, K).to(torch.int8)
+    return _fragments_to_logical(act, M_pad, K, ACT_BLOCK_ROWS)
+
+
+def _fragments_to_logical(buf: torch.Tensor, rows: int, K: int, block_rows: int) -> torch.Tensor:
+    """E2M3 fragments ``[rows/block_rows][K/64][block_rows/32]`` -> int8 codes [rows, K]."""
+    import numpy as np
+
+    nf = block_rows // 32
+    f = buf.contiguous().cpu().view(torch.uint8).reshape(rows // block_rows, K // 64, nf, FRAG_BYTES)
+    strings = torch.cat([f[..., :1024].reshape(*f.shape[:3], 64, 16), f[..., 1024:].reshape(*f.shape[:3], 64, 8)], dim=-1)
+    bits = np.unpackbits(strings.numpy(), axis=-1, bitorder="little").reshape(*f.shape[:3], 64, 32, 6)
+    pat = (bits * np.array([1, 2, 4, 8, 16, 32], dtype=np.uint8)).sum(axis=-1).astype(np.int64)  # [blk, g, frag, slot, 32]
+    codes = _E2M3_TO_CODE[torch.from_numpy(pat)]
+    assert (codes != 127).all(), "a pattern that is not code / 2 for any INT4 code"
+    # slot = row + 32 * half, element j of a half is column 32 * half + j
+    codes = codes.reshape(rows // block_rows, K // 64, nf, 2, 32, 32).permute(0, 2, 4, 1, 3, 5)  # blk, frag, row, g, half, j
+    return codes.reshape(rows, K).contiguous().to(buf.device)
+
+
+def qweight_to_logical(qweight_native: torch.Tensor) -> torch.Tensor:
+    """Native INT4 weights (``repack_qweight``) -> int8 codes [N, K] (tests and debugging)."""
+    N, K = qweight_native.logical_shape
+    return _fragments_to_logical(qweight_native, qweight_native.shape[0], K, WGT_BLOCK_COLS)[:N]
+
+
+def wscales_to_logical(wscales_native: torch.Tensor, N: int) -> torch.Tensor:
+    """Native INT4 weight scales (``repack_wscales``) -> fp32 [K/64, N] (the factor 4 taken out again)."""
+    w = wscales_native.cpu()  # int64 [nblocks, G, 256], bf16 bits of 4 * scale in the low 16 bits
+    assert ((w >> 16) == 0).all(), "the upper three 16-bit slots of a scale entry must be zero"
+    v = (w.to(torch.int32) << 16).view(torch.float32) * 0.25
+    return v.permute(1, 0, 2).reshape(w.shape[1], -1)[:, :N].contiguous()
 
 
 def logical_to_act(codes: torch.Tensor, fp4: bool = False, unsigned: bool = False) -> torch.Tensor:
     """Inverse of :func:`act_to_logical` (used by tests to feed hand-made codes to the GEMM)."""
     M_pad, K = codes.shape
-    c = codes.to(torch.int64)
-    if not fp4 and not unsigned:
-        c = c + 8
-    c = (c & 0xF).reshape(M_pad // 32, 32, K // 64, 8, 8).permute(0, 2, 1, 3, 4)  # tile, group, row, word, element
-    w = sum(c[..., e] << (4 * e) for e in range(8))
-    if not fp4:
-        w = ((w << INT4_WORD_ROT) | (w >> (32 - INT4_WORD_ROT))) & 0xFFFFFFFF
-    w = torch.where(w >= 2**31, w - 2**32, w).to(torch.int32)
-    return w.contiguous().view(torch.uint8).reshape(M_pad, K // 2)
+    if fp4:
+        c = (codes.to(torch.int64) & 0xF).reshape(M_pad // 32, 32, K // 64, 8, 8).permute(0, 2, 1, 3, 4)  # tile, group, row, word, element
+        w = sum(c[..., e] << (4 * e) for e in range(8))
+        w = torch.where(w >= 2**31, w - 2**32, w).to(torch.int32)
+        return w.contiguous().view(torch.uint8).reshape(M_pad, K // 2)
+    import numpy as np
+
+    pat = _CODE_TO_E2M3[codes.cpu().to(torch.int64) + 16]
+    pat = pat.reshape(M_pad // ACT_BLOCK_ROWS, 4, 32, K // 64, 2, 32).permute(0, 3, 1, 4, 2, 5)  # blk, g, frag, half, row, j
+    pat = pat.reshape(M_pad // ACT_BLOCK_ROWS, K // 64, 4, 64, 32).numpy()
+    bits = ((pat[..., None] >> np.arange(6, dtype=np.uint8)) & 1).astype(np.uint8).reshape(*pat.shape[:4], 192)
+    strings = torch.from_numpy(np.packbits(bits, axis=-1, bitorder="little"))  # [blk, g, frag, slot, 24]
+    f = torch.cat([strings[..., :16].reshape(*pat.shape[:3], 1024), strings[..., 16:].reshape(*pat.shape[:3], 512)], dim=-1)
+    return f.reshape(M_pad, K * 3 // 4).contiguous().to(codes.device)
 
 
 def scales_to_logical(scales: torch.Tensor, fp4: bool = False) -> torch.Tensor:

@@ -31,7 +31,7 @@ def test_header_symbols_are_exported(lib):
 
 def test_struct_sizes_match_header_layout():
     # 6 pointers + 4 int64 + 2 int32 ; 16 pointers + 7 int64 + float + 3 int32, then 3 pointers + int64 +
-    # float (padded to 8)
+    # float + int32
     assert ctypes.sizeof(nv.QuantizeArgs) == 6 * 8 + 4 * 8 + 2 * 4
     assert ctypes.sizeof(nv.GemmArgs) == 16 * 8 + 7 * 8 + 4 * 4 + 3 * 8 + 8 + 8
 
@@ -84,13 +84,16 @@ def test_gemm_rejects_bad_arguments(lib):
     bad.oscales = 16
     bad.next_smooth_rcp = 16
     assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
-    # INT4 takes neither a per-tensor scale nor per-channel scales (NVFP4 only)
     bad = nv.GemmArgs.from_buffer_copy(a)
-    bad.alpha = 0.5
-    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
+    bad.k_split = -1
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
     bad = nv.GemmArgs.from_buffer_copy(a)
-    bad.wcscales = 16
-    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -2
+    bad.fp4 = 1
+    bad.colnorm = None  # NVFP4 needs the column factors of its repack
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
+    bad = nv.GemmArgs.from_buffer_copy(a)
+    bad.R_down = 32  # without next_lora_down / next_lora_act_out
+    assert lib.svdq_gemm_w4a4(ctypes.byref(bad), None) == -1
     # the norm + rotary epilogue: needs both norm weights, three equal parts of whole heads, enough table rows
     bad = nv.GemmArgs.from_buffer_copy(a)
     bad.norm_q = 16
@@ -119,7 +122,8 @@ def test_repack_rejects_bad_arguments(lib):
     assert lib.svdq_repack_qweight(None, None, 128, 128, 0, None) == -1
     assert lib.svdq_repack_qweight(16, 32, 100, 128, 0, None) == -1
     assert lib.svdq_repack_qweight(16, 16, 128, 128, 0, None) == -1  # in place
-    assert lib.svdq_repack_wscales(16, 32, 48, 128, 100, None) == -1
+    assert lib.svdq_repack_wscales(16, 32, 128, 100, None) == -1
+    assert lib.svdq_repack_wscales(16, 40, 128, 128, None) == -1  # destination not 16-byte aligned
     assert lib.svdq_repack_vector(16, 32, 100, None) == -1
     assert lib.svdq_repack_smooth(16, 32, 64, None) == -1
     assert lib.svdq_repack_lora_down(16, 32, 128, 8, None) == -1
@@ -169,11 +173,125 @@ def test_module_mirrors_reference_parameters():
     assert SVDQW4A4Linear.from_linear(lin, rank=16).rank == 16
 
 
-def test_probe_library_exports_its_entry_point():
-    """bench.py's MFMA-rate probe is a library of its own (not part of the operator ABI); no GPU call here."""
-    import ctypes
+def test_gemm_wrapper_refuses_wrong_shapes(monkeypatch):
+    """Every buffer the kernel walks over M_pad rows of is checked before anything is launched (an
+    undersized one would be an out-of-bounds access on the device).  No GPU: the device check is
+    switched off so that the shape checks are reached with CPU tensors."""
+    import torch
 
-    from nunchaku_amd import _native as nv
+    from nunchaku_amd import packing
+    from nunchaku_amd.ops import gemm as gemm_mod
 
-    assert nv.PROBE_LIB_PATH.exists(), "build with __graft_entry__.build()"
-    assert hasattr(ctypes.CDLL(str(nv.PROBE_LIB_PATH)), "svdq_probe_mfma_rate")
+    monkeypatch.setattr(nv, "require_gpu", lambda t, name: None)
+
+    def boom(*a, **k):
+        raise AssertionError("reached the repack / launch")
+
+    monkeypatch.setattr(packing, "native", boom)
+    M_pad, K, N, R = 256, 128, 128, 16
+    good = dict(
+        act=torch.zeros(M_pad, K * 3 // 4, dtype=torch.uint8), wgt=torch.zeros(N, K // 2, dtype=torch.int8),
+        ascales=torch.zeros(K // 64, M_pad, dtype=torch.bfloat16), wscales=torch.zeros(K // 64, N, dtype=torch.bfloat16),
+        out=torch.zeros(M_pad, N, dtype=torch.bfloat16), lora_act_in=torch.zeros(M_pad, R), lora_up=torch.zeros(N, R, dtype=torch.bfloat16),
+        bias=torch.zeros(N, dtype=torch.bfloat16),
+    )
+    with pytest.raises(AssertionError, match="reached"):
+        gemm_mod.svdq_gemm_w4a4(**good)  # (the valid call gets as far as the repack)
+    cases = {
+        "act": torch.zeros(M_pad, K // 2, dtype=torch.uint8),           # the reference's 4-bit shape
+        "ascales": torch.zeros(K // 64, 100, dtype=torch.bfloat16),     # unpadded
+        "wscales": torch.zeros(K // 64, N + 1, dtype=torch.bfloat16),
+        "lora_act_in": torch.zeros(100, R),                             # [M, R] instead of [M_pad, R]
+        "lora_up": torch.zeros(N - 16, R, dtype=torch.bfloat16),
+        "bias": torch.zeros(N, dtype=torch.float32),
+    }
+    for name, t in cases.items():
+        with pytest.raises(ValueError, match=name):
+            gemm_mod.svdq_gemm_w4a4(**{**good, name: t})
+    nxt = dict(qout=torch.zeros(M_pad, N * 3 // 4, dtype=torch.uint8), oscales=torch.zeros(N // 64, M_pad, dtype=torch.bfloat16),
+               smooth_factor=torch.ones(N, dtype=torch.bfloat16), lora_down=torch.zeros(N, R, dtype=torch.bfloat16), lora_act_out=torch.zeros(M_pad, R))
+    for name, t in {"qout": torch.zeros(M_pad, N // 2, dtype=torch.uint8), "oscales": torch.zeros(N // 64, 128, dtype=torch.bfloat16),
+                    "lora_act_out": torch.zeros(128, R), "smooth_factor": torch.ones(N - 1, dtype=torch.bfloat16)}.items():
+        with pytest.raises(ValueError, match=name):
+            gemm_mod.svdq_gemm_w4a4(**{**good, **nxt, name: t})
+
+
+def test_quantize_wrapper_refuses_wrong_shapes(monkeypatch):
+    import torch
+
+    from nunchaku_amd.ops import svdq_quantize_w4a4_act_fuse_lora
+
+    monkeypatch.setattr(nv, "require_gpu", lambda t, name: None)
+    x = torch.zeros(100, 128, dtype=torch.bfloat16)
+    down = torch.zeros(128, 16, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="output"):
+        svdq_quantize_w4a4_act_fuse_lora(x, output=torch.zeros(256, 64, dtype=torch.uint8), lora_down=down)
+    with pytest.raises(ValueError, match="oscales"):
+        svdq_quantize_w4a4_act_fuse_lora(x, oscales=torch.zeros(2, 100, dtype=torch.bfloat16), lora_down=down)
+    with pytest.raises(ValueError, match="lora_act_out"):
+        svdq_quantize_w4a4_act_fuse_lora(x, lora_act_out=torch.zeros(100, 16), lora_down=down)
+    with pytest.raises(ValueError, match="lora_down"):
+        svdq_quantize_w4a4_act_fuse_lora(x, lora_down=torch.zeros(64, 16, dtype=torch.bfloat16))
+
+
+def test_repack_cache_follows_modifications(monkeypatch):
+    """The cache of repacked reference tensors: hit while the source is unchanged, redone after an
+    in-place operation, and tensors without a version counter (inference mode) are never cached."""
+    import torch
+
+    from nunchaku_amd import packing
+
+    calls = []
+
+    def fake(t):
+        calls.append(t)
+        return t.clone()
+
+    monkeypatch.setitem(packing._REPACKERS, "vector", fake)
+    t = torch.ones(128, dtype=torch.bfloat16)
+    a = packing.native(t, "vector")
+    assert packing.native(t, "vector") is a and len(calls) == 1
+    t.add_(1)
+    assert packing.native(t, "vector") is not a and len(calls) == 2
+    with torch.inference_mode():
+        u = torch.ones(128, dtype=torch.bfloat16)
+    assert packing.tensor_version(u) is None
+    packing.native(u, "vector")
+    packing.native(u, "vector")
+    assert len(calls) == 4
+
+
+def test_module_reconverts_after_a_parameter_changes(monkeypatch):
+    """A low-rank swap or any other in-place update of a parameter is picked up by the next forward."""
+    import torch
+
+    from nunchaku_amd import packing
+    from nunchaku_amd.models.linear import SVDQW4A4Linear
+
+    count = {"n": 0}
+
+    def fake(t, *a):
+        count["n"] += 1
+        return t.clone()
+
+    for name in ("repack_qweight", "repack_wscales", "repack_smooth", "repack_lora_down", "repack_lora_up", "repack_vector"):
+        monkeypatch.setattr(packing, name, fake)
+    m = SVDQW4A4Linear(128, 128, rank=16)
+    for p in m.parameters():
+        p.data.zero_()
+    m.native_tensors()
+    n0 = count["n"]
+    assert m.native_tensors() is m.native_tensors() and count["n"] == n0
+    with torch.no_grad():
+        m.proj_up.add_(1)  # in place: the version counter moves
+    m.native_tensors()
+    assert count["n"] == 2 * n0
+    m.proj_up = torch.nn.Parameter(torch.zeros(128, 32, dtype=torch.bfloat16))  # replaced (rank growth)
+    m.native_tensors()
+    assert count["n"] == 3 * n0
+    m.proj_up.data.copy_(torch.ones(128, 32))  # leaves no trace: needs the explicit call
+    m.native_tensors()
+    assert count["n"] == 3 * n0
+    m.invalidate_native()
+    m.native_tensors()
+    assert count["n"] == 4 * n0

@@ -35,7 +35,7 @@ def test_next_layer_epilogue(dev, M, K1, N1, N2, R):
     qx, asc, la = m1.quantize(x.to(dev))
     M_pad = qx.shape[0]
     out = torch.empty(M_pad, N1, dtype=torch.bfloat16, device=dev)
-    qout = torch.empty(M_pad, N1 // 2, dtype=torch.uint8, device=dev)
+    qout = torch.empty(M_pad, N1 * 3 // 4, dtype=torch.uint8, device=dev)
     osc = torch.empty(N1 // 64, M_pad, dtype=torch.bfloat16, device=dev)
     la2 = torch.full((M_pad, R), float("nan"), dtype=torch.float32, device=dev)
     svdq_gemm_w4a4(act=qx, wgt=t1["qweight"], out=out, qout=qout, ascales=asc, wscales=t1["wscales"], oscales=osc,
@@ -92,7 +92,7 @@ def test_mlp_flux_shape(dev):
     t1, t2 = m1.native_tensors(), m2.native_tensors()
     qx, asc, la = m1.quantize(x.to(dev))
     out = torch.empty(M, c1["N"], dtype=torch.bfloat16, device=dev)
-    qout = torch.empty(M, c1["N"] // 2, dtype=torch.uint8, device=dev)
+    qout = torch.empty(M, c1["N"] * 3 // 4, dtype=torch.uint8, device=dev)
     osc = torch.empty(c1["N"] // 64, M, dtype=torch.bfloat16, device=dev)
     la2 = torch.empty(M, c2["R"], dtype=torch.float32, device=dev)
     svdq_gemm_w4a4(act=qx, wgt=t1["qweight"], out=out, qout=qout, ascales=asc, wscales=t1["wscales"], oscales=osc,

@@ -160,3 +160,32 @@ def test_fuse_silu_epilogue(dev):
     check_output(out, want)
     plain = m.forward_quant(qx, asc, la)[:M]  # not the identity: the plain output differs
     assert not torch.equal(plain, out)
+
+
+def test_gemm_int4_per_channel_scales_and_alpha(dev):
+    """INT4 with ``wcscales`` and ``alpha`` (EpilogueBias<.., USE_SCALE>, gemm_w4a4_launch_impl.cuh:174-187):
+    both multiply the main term only, the bias and the low-rank term are added after."""
+    from nunchaku_amd import packing
+    from nunchaku_amd.ops import svdq_gemm_w4a4
+
+    M, K, N, R = 256, 256, 384, 32
+    announce(f"gemm INT4 wcscales + alpha M={M} K={K} N={N}")
+    layer = synth.make_layer(N, K, R, seed=77)
+    g = torch.Generator().manual_seed(77)
+    codes = torch.randint(-8, 8, (M, K), generator=g).to(torch.int8)
+    scales = (torch.rand(K // 64, M, generator=g) * 0.5 + 0.01).to(torch.bfloat16)
+    lora_act = torch.randn(M, R, generator=g) * 3
+    wcs = (0.25 + 2 * torch.rand(N, generator=g)).to(torch.bfloat16)
+    wcs[5] = 0.0  # a zero per-channel scale leaves bias + low-rank term
+    m = make_module(layer, dev)
+    t = m.native_tensors()
+    for alpha in (1.0, 0.625):
+        out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        svdq_gemm_w4a4(act=packing.logical_to_act(codes).to(dev), wgt=t["qweight"], out=out, ascales=scales.to(dev), wscales=t["wscales"],
+                       lora_act_in=lora_act.to(dev), lora_up=t["proj_up"], bias=t["bias"], wcscales=packing.repack_vector(
+                           torch.from_numpy(__import__("oracle.layouts", fromlist=["x"]).pack_vector(wcs.view(torch.int16).numpy().view("uint16")).view("int16").copy()).view(torch.bfloat16).to(dev)),
+                       alpha=alpha)
+        torch.cuda.synchronize()
+        want = olin.gemm_w4a4(quant.dequant_int4(codes, scales), quant.dequant_int4(layer.wq, layer.ws), bias=layer.bias,
+                              lora_act_in=lora_act, lora_up=layer.proj_up, alpha=alpha, wcscales=wcs)
+        check_output(out, want)

@@ -25,15 +25,12 @@ def test_repack_golden_vectors(dev):
     announce("repack golden qweight/wscales/vector/lora N=K=256 R=32")
     qn = packing.repack_qweight(torch.from_numpy(z["qweight"]).to(dev))
     N, K = z["codes"].shape
-    # native tiles hold offset-binary codes in row/column order
-    assert torch.equal(packing.act_to_logical(qn.view(torch.uint8).cpu(), K), torch.from_numpy(z["codes"]))
+    # E2M3 fragments of code / 2, decoded back to one code per element
+    assert torch.equal(packing.qweight_to_logical(qn).cpu(), torch.from_numpy(z["codes"]))
 
     ws = packing.repack_wscales(_bf16(z["wscales_packed"]).to(dev))
     logical = _bf16(z["wscales_logical"]).float()
-    back = ws.float().cpu() * ws.colnorm.cpu()[None, :]
-    assert torch.equal(back, logical)  # power-of-two normalisation is exact
-    amax = ws.float().abs().amax(dim=0).cpu()
-    assert ((amax >= 1024) & (amax < 2048)).all()
+    assert torch.equal(packing.wscales_to_logical(ws, N), logical)  # the factor 4 is a power of two: exact
 
     v = packing.repack_vector(_bf16(z["vec_packed"].reshape(-1)).to(dev))
     assert torch.equal(v.cpu().view(torch.int16), _bf16(z["vec_logical"]).view(torch.int16))
@@ -76,7 +73,15 @@ def test_repack_random_larger(dev):
     announce(f"repack random N={N} K={K}")
     codes = rng.integers(-8, 8, (N, K)).astype(np.int8)
     qn = packing.repack_qweight(torch.from_numpy(L.pack_qweight(codes)).to(dev))
-    assert torch.equal(packing.act_to_logical(qn.view(torch.uint8).cpu(), K), torch.from_numpy(codes))
+    assert torch.equal(packing.qweight_to_logical(qn).cpu(), torch.from_numpy(codes))
+    assert qn.shape == (512, K * 3 // 4), "N = 384 is padded to two blocks of 256 columns"
+    pad = packing._fragments_to_logical(qn, 512, K, 256)[N:]
+    assert (pad == 0).all(), "columns beyond N must hold zero codes"
+    ws = rng.random((K // 64, N)).astype(np.float32) + 0.01
+    wsb = torch.from_numpy(ws).to(torch.bfloat16)
+    wn = packing.repack_wscales(torch.from_numpy(L.pack_wscales(wsb.view(torch.int16).numpy().view(np.uint16)).view(np.int16).copy()).view(torch.bfloat16).to(dev))
+    assert torch.equal(packing.wscales_to_logical(wn, N), wsb.float())
+    assert (wn.cpu()[1, :, 128:] == 0).all(), "scales of the columns beyond N must be zero"
     pat = rng.integers(0, 16, (N, K)).astype(np.int8)
     qf = packing.repack_qweight(torch.from_numpy(L.pack_qweight(pat)).to(dev), fp4=True)
     assert torch.equal(packing.act_to_logical(qf.view(torch.uint8).cpu(), K, fp4=True), torch.from_numpy(pat))
