@@ -104,54 +104,62 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
 
     // ---- which tile, which part of its k-groups ------------------------------------------------
-    // Workgroups go to the XCDs round robin (blockIdx % 8); the remap gives each XCD one contiguous
-    // run of tiles, numbered down M first, so that the workgroups resident on an XCD at one time share
-    // their weight columns and their activation rows in that XCD's L2.
-    const int mblocks = p.M_pad / BM;
+    // Workgroups go to the XCDs round robin (blockIdx % 8); the remap gives each XCD one contiguous run
+    // of tile numbers, and the tiles are numbered in bands of 16 row blocks, down the band first: the 64
+    // workgroups resident on an XCD at one time then cover about 16 row blocks x 4 column blocks, whose
+    // operands (6 KB per row block and k-group, 14 KB per column block) they share in that XCD's L2.
+    const int mblocks = p.M_pad / BM, nblocks = (p.N + BN - 1) / BN;
     const int kgroups = p.K / 64;
     const int total = (int)gridDim.x;
     int v = (int)blockIdx.x;
     if (total % 8 == 0) v = (v % 8) * (total / 8) + v / 8;
     const int tile = v / p.kparts, part = v - tile * p.kparts;
-    const int mb = tile % mblocks, nb = tile / mblocks;
+    constexpr int BAND = 16;
+    const int band = tile / (BAND * nblocks), in_band = tile - band * (BAND * nblocks);
+    const int band_rows = mblocks - band * BAND < BAND ? mblocks - band * BAND : BAND;
+    const int mb = band * BAND + in_band % band_rows, nb = in_band / band_rows;
     const int gb = (int)((long long)kgroups * part / p.kparts);
     const int ng = (int)((long long)kgroups * (part + 1) / p.kparts) - gb;
     const int m0 = mb * BM, n0 = nb * BN;
 
     // ---- staging ---------------------------------------------------------------------------------
-    // Every wave issues COPIES_PER_WAVE copies per k-group: three 1 KB chunks of the weight fragments,
-    // one of the activation fragments, one more of those (waves 0, 1) or of the weight scales (waves
-    // 2, 3), and the 256 bytes of activation scales (all four waves write the same bytes: the counts
-    // stay equal, which keeps the wait below a constant).
+    // Every wave issues COPIES_PER_WAVE copies per k-group: three consecutive 1 KB chunks of the weight
+    // fragments (one base, the instruction's offset field advances both the memory and the LDS address),
+    // one chunk of the activation fragments, one more of those (waves 0, 1) or of the weight scales
+    // (waves 2, 3), and the 256 bytes of activation scales (all four waves write the same bytes: the
+    // counts stay equal, which keeps the wait below a constant).  The four source pointers are
+    // wave-uniform and advance by a constant per k-group.
     const uint32_t copy_voff = lane * 16;
-    auto issue_copies = [&](int l) {  // l counts this workgroup's k-groups
-        const int g = gb + l;
-        const uint32_t dst = lds_base + (l % STAGES) * STAGE_BYTES;
-        const uint8_t *wsrc = p.wgt + ((size_t)nb * kgroups + g) * (8 * FRAG_BYTES);
-        const uint8_t *asrc = p.act + ((size_t)mb * kgroups + g) * (4 * FRAG_BYTES);
-        const uint8_t *ssrc = p.wscales + ((size_t)nb * kgroups + g) * 2048;
-        const uint8_t *qsrc = (const uint8_t *)(p.ascales + (size_t)g * p.M_pad + m0);
-#pragma unroll
-        for (int i = 0; i < 3; i++)
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :: "s"(dst + ST_W + (wave + 4 * i) * 1024), "v"(copy_voff), "s"(wsrc + (wave + 4 * i) * 1024) : "memory");
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(dst + ST_A + wave * 1024), "v"(copy_voff), "s"(asrc + wave * 1024) : "memory");
-        const bool low = wave < 2;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(dst + (low ? ST_A + (4 + wave) * 1024 : ST_WS + (wave - 2) * 1024)), "v"(copy_voff),
-                        "s"(low ? asrc + (4 + wave) * 1024 : ssrc + (wave - 2) * 1024) : "memory");
+    const bool low = wave < 2;
+    const uint8_t *src_w = p.wgt + ((size_t)nb * kgroups + gb) * (8 * FRAG_BYTES) + wave * 3072;
+    const uint8_t *src_a = p.act + ((size_t)mb * kgroups + gb) * (4 * FRAG_BYTES) + wave * 1024;
+    const uint8_t *src_x = low ? p.act + ((size_t)mb * kgroups + gb) * (4 * FRAG_BYTES) + (4 + wave) * 1024
+                               : p.wscales + ((size_t)nb * kgroups + gb) * 2048 + (wave - 2) * 1024;
+    const uint8_t *src_q = (const uint8_t *)(p.ascales + (size_t)gb * p.M_pad + m0);
+    const uint32_t stride_x = low ? 4 * FRAG_BYTES : 2048, stride_q = (uint32_t)p.M_pad * 2;
+    const uint32_t dst_w = lds_base + ST_W + wave * 3072, dst_a = lds_base + ST_A + wave * 1024;
+    const uint32_t dst_x = lds_base + (low ? ST_A + (4 + wave) * 1024 : ST_WS + (wave - 2) * 1024), dst_q = lds_base + ST_AS;
+    auto issue_copies = [&](uint32_t stage_off) {  // the next k-group not yet requested, into the stage at stage_off
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %2, %3\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024\n\tglobal_load_lds_dwordx4 %2, %3 offset:2048"
+                     :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_a), "s"(stage_off), "v"(copy_voff), "s"(src_a) : "memory");
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_x), "s"(stage_off), "v"(copy_voff), "s"(src_x) : "memory");
         uint32_t voff4;
         asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(voff4) : "v"(copy_voff));
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" :: "s"(dst + ST_AS), "v"(voff4), "s"(qsrc) : "memory");
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3" :: "s"(dst_q), "s"(stage_off), "v"(voff4), "s"(src_q) : "memory");
+        src_w += 8 * FRAG_BYTES;
+        src_a += 4 * FRAG_BYTES;
+        src_x += stride_x;
+        src_q += stride_q;
     };
 
     // what the upper half-wave reads as its activation scale
     if (tid < STAGES * 32) *(uint32_t *)(lds + (tid >> 5) * STAGE_BYTES + ST_Z + (tid & 31) * 4) = 0u;
 
     issue_copies(0);
-    if (ng > 1) issue_copies(1);
-    if (ng > 2) issue_copies(2);
+    if (ng > 1) issue_copies(STAGE_BYTES);
+    if (ng > 2) issue_copies(2 * STAGE_BYTES);
 
     // per-lane read offsets inside a stage
     const uint32_t off16 = lane * 16, off8 = 1024 + lane * 8;
@@ -216,7 +224,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     // below the branch, with all their operands alive).  BULK: the groups that still have copies to
     // request (l + 3 < ng); the last three groups run the same body without requests and wait for
     // everything outstanding.
-    auto group_body = [&](int l, auto BULK_T) {
+    auto group_body = [&](auto BULK_T) {
         constexpr bool BULK = decltype(BULK_T)::value;
         const uint32_t sb_next = sb == (STAGES - 1) * STAGE_BYTES ? 0 : sb + STAGE_BYTES;
         // step t issues the matrix instructions of tile t + 1 (tile = 2 nt + mt) and accumulates tile t
@@ -233,7 +241,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         // stage, whose copies every wave has waited for, may be read.
         if (BULK) {
             asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            issue_copies(l + 3);
+            issue_copies(sb);  // group l + 3 into the stage of group l
         } else {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
@@ -247,8 +255,8 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         sb = sb_next;
     };
     int l = 0;
-    for (; l + 3 < ng; l++) group_body(l, std::true_type{});
-    for (; l < ng; l++) group_body(l, std::false_type{});
+    for (; l + 3 < ng; l++) group_body(std::true_type{});
+    for (; l < ng; l++) group_body(std::false_type{});
 #undef SVDQ_STEP
 #undef SVDQ_FMA
     __syncthreads();  // the ring is free: the epilogue reuses it
