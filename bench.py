@@ -72,6 +72,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="flux_mlp_fc1", choices=sorted(WORKLOADS))
+    ap.add_argument("--shape", default=None, help="M,K,N,R of an INT4 layer to time instead of a named workload (seed 9)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=4608)
     ap.add_argument("--qkv-rope", action="store_true",
@@ -151,6 +152,10 @@ def main():
     from oracle import synth
 
     cfg = WORKLOADS[args.workload]
+    if args.shape:
+        m_, k_, n_, r_ = (int(v) for v in args.shape.split(","))
+        cfg = dict(M=m_, K=k_, N=n_, R=r_, seed=9)
+        args.workload = f"custom_{m_}x{k_}x{n_}_r{r_}"
     M, K, N, R = cfg["M"], cfg["K"], cfg["N"], cfg["R"]
     dev = torch.device("cuda:0")
     fp4 = bool(cfg.get("fp4"))
