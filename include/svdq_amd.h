@@ -184,6 +184,19 @@ typedef struct svdq_gemm_args {
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
 
+/* The same operator for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  It runs the
+ * same kernels as svdq_gemm_w4a4 and gives the same results bit for bit, but calls that need a workspace
+ * (see above) take it from a fixed array in device memory (42 MB on every GPU the library runs on, held
+ * until the process ends: 10 MB for arrival counters and fixed-point sums, 32 MB for partial sums) instead
+ * of allocating one: no hipMalloc, hipFree or other allocating call is made.  A call whose need exceeds
+ * the array returns SVDQ_EUNSUPPORTED with a message that says how much it wanted (examples that fit:
+ * INT4 M_pad = 256, K = N = 3072 split six ways, 18.9 MB of partial sums; next_lora_down with M_pad * R_down
+ * up to 1.3 M elements).  All calls on one GPU share the array, whatever their stream: calls that overlap
+ * in time on one GPU race with each other.  What a launch needs to be zero at its start is cleared by a
+ * fill kernel on `stream` first. */
+int svdq_gemm_w4a4_noalloc(const svdq_gemm_args *args, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * AWQ W4A16 GEMV (the other quantized linear of the reference's models: modulation layers, text
  * encoder), for 1..8 rows of x.  Replaces ops.gemv_awq (nunchaku/ops/gemv.py ->

@@ -29,7 +29,7 @@ EXPORTED_SYMBOLS = [
     "svdq_abi_version", "svdq_last_error",
     "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
     "svdq_repack_smooth", "svdq_repack_lora_down", "svdq_repack_lora_up", "svdq_repack_rotemb",
-    "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4", "svdq_awq_gemv_w4a16",
+    "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4", "svdq_gemm_w4a4_noalloc", "svdq_awq_gemv_w4a16",
 ]
 
 
@@ -136,6 +136,7 @@ def lib() -> ctypes.CDLL:
         L.svdq_repack_rotemb.argtypes = [vp, vp, i64, vp]
         L.svdq_quantize_w4a4_act_fuse_lora.argtypes = [ctypes.POINTER(QuantizeArgs), vp]
         L.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.svdq_gemm_w4a4_noalloc.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), vp]
         for name in EXPORTED_SYMBOLS:
             getattr(L, name)

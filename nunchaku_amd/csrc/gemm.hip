@@ -86,6 +86,65 @@ Workspace *get_workspace(int dev, hipStream_t stream, size_t zero_bytes, size_t 
     return w;
 }
 
+// ---- the scratch of svdq_gemm_w4a4_noalloc --------------------------------------------------------
+// A fixed array in device memory, one copy per GPU, held until the process ends: first the region that
+// must be zero when a launch starts (arrival counters, fixed-point sums), then parked partial sums.
+constexpr size_t NOALLOC_ZERO_BYTES = 10u << 20, NOALLOC_SCRATCH_BYTES = 32u << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_ZERO_BYTES + NOALLOC_SCRATCH_BYTES];
+uint8_t *g_scratch_ptr[64] = {nullptr};  // the array's device address on each GPU, asked once per GPU
+std::mutex g_scratch_mutex;
+
+// the array's address on device `dev` (which is the current device), or nullptr with the error text set
+uint8_t *scratch_address(int dev) {
+    if (dev < 0 || dev >= 64) {
+        fail(SVDQ_ELAUNCH, "gemm: device index %d out of range", dev);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            fail(SVDQ_ELAUNCH, "gemm: cannot locate the scratch array on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = (uint8_t *)ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
+// Where a launch gets its workspace from: the per-(device, stream) allocation of svdq_gemm_w4a4, or the
+// fixed scratch array of svdq_gemm_w4a4_noalloc.
+struct WorkspaceView {
+    uint8_t *zero;     // zero_bytes that are zero when the launch starts
+    uint8_t *scratch;  // scratch_bytes of anything
+    Workspace *owner;  // the allocation behind it (nullptr for the fixed array)
+};
+
+// (the caller holds g_ws_mutex when `noalloc` is false) false, with the error text set, on failure
+bool acquire_workspace(bool noalloc, int dev, hipStream_t st, size_t zero_bytes, size_t scratch_bytes, WorkspaceView *v) {
+    if (!noalloc) {
+        Workspace *w = get_workspace(dev, st, zero_bytes, scratch_bytes);
+        if (!w) return false;
+        *v = WorkspaceView{w->ptr, w->ptr + w->zero_bytes, w};
+        return true;
+    }
+    if (zero_bytes > NOALLOC_ZERO_BYTES || scratch_bytes > NOALLOC_SCRATCH_BYTES) {
+        fail(SVDQ_EUNSUPPORTED, "gemm (noalloc): this call needs %zu + %zu bytes of workspace, the fixed scratch holds %zu + %zu; use svdq_gemm_w4a4",
+             zero_bytes, scratch_bytes, NOALLOC_ZERO_BYTES, NOALLOC_SCRATCH_BYTES);
+        return false;
+    }
+    uint8_t *base = scratch_address(dev);
+    if (!base) return false;
+    // The array keeps the last call's contents.  A launch that completes leaves its counters and sums at
+    // zero, one that failed or was aborted does not: what this launch needs to be zero is cleared (by a
+    // fill kernel, which a caller's graph capture can record).
+    const int64_t n = (int64_t)((zero_bytes + 15) / 16 * 4);
+    if (n > 0) hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, (float *)base, n);
+    *v = WorkspaceView{base, base + NOALLOC_ZERO_BYTES, nullptr};
+    return true;
+}
+
 // number of compute units of a device, asked once
 int compute_units(int dev) {
     static int cached[64] = {0};
@@ -99,7 +158,7 @@ int compute_units(int dev) {
 }
 
 // ---- INT4: fp6 matrix instruction on the bare codes (gemm6_kernel.h) --------------------------------
-int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu) {
+int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noalloc) {
     g6::Params p;
     p.act = (const uint8_t *)a->act;
     p.ascales = (const uint16_t *)a->ascales;
@@ -151,21 +210,22 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu) {
     const size_t fix_bytes = p.next_down ? (size_t)p.M_pad * p.R_down * 8 : 0;
     const size_t part_bytes = kparts > 1 ? (size_t)ntiles * kparts * g6::BM * g6::BN * 4 : 0;
     if (kparts == 1 && !p.next_down) return next ? g6::launch_next(p, ntiles, st) : g6::launch_plain(p, ntiles, st);
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
+    if (!noalloc) lock.lock();
     const size_t cnt_pad = (cnt_bytes + lcnt_bytes + 255) & ~(size_t)255;
-    Workspace *w = get_workspace(dev, st, cnt_pad + fix_bytes, part_bytes);
-    if (!w) return SVDQ_ELAUNCH;
-    p.counters = (int *)w->ptr;
-    p.next_lora_cnt = (int *)(w->ptr + cnt_bytes);
-    p.next_lora_fix = (long long *)(w->ptr + cnt_pad);
-    p.partials = (float *)(w->ptr + w->zero_bytes);
+    WorkspaceView w;
+    if (!acquire_workspace(noalloc, dev, st, cnt_pad + fix_bytes, part_bytes, &w)) return noalloc && (cnt_pad + fix_bytes > NOALLOC_ZERO_BYTES || part_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
+    p.counters = (int *)w.zero;
+    p.next_lora_cnt = (int *)(w.zero + cnt_bytes);
+    p.next_lora_fix = (long long *)(w.zero + cnt_pad);
+    p.partials = (float *)w.scratch;
     const int rc = next ? g6::launch_next(p, ntiles * kparts, st) : g6::launch_plain(p, ntiles * kparts, st);
-    if (rc != SVDQ_OK) w->dirty = true;
+    if (rc != SVDQ_OK && w.owner) w.owner->dirty = true;
     return rc;
 }
 
 // ---- NVFP4: fp16 matrix instruction on dequantized operands (gemm_kernel.h) -------------------------
-int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu) {
+int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noalloc) {
     GemmParams p;
     p.act = (const uint8_t *)a->act;
     p.ascales = (const uint16_t *)a->ascales;
@@ -221,18 +281,21 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu) {
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, p.next_lora_out, n);
     }
     if (nwg <= ntiles && ntiles % nwg == 0) return next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace *w = get_workspace(dev, st, (size_t)ntiles * 4, (size_t)2 * nwg * 256 * 64 * 16);
-    if (!w) return SVDQ_ELAUNCH;
-    p.counters = (int *)w->ptr;
-    p.partials = (float *)(w->ptr + w->zero_bytes);
+    std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
+    if (!noalloc) lock.lock();
+    const size_t zero_bytes = (size_t)ntiles * 4, part_bytes = (size_t)2 * nwg * 256 * 64 * 16;
+    WorkspaceView w;
+    if (!acquire_workspace(noalloc, dev, st, zero_bytes, part_bytes, &w)) return noalloc && (zero_bytes > NOALLOC_ZERO_BYTES || part_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
+    p.counters = (int *)w.zero;
+    p.partials = (float *)w.scratch;
     const int rc = next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
-    if (rc != SVDQ_OK) w->dirty = true;
+    if (rc != SVDQ_OK && w.owner) w.owner->dirty = true;
     return rc;
 }
 }  // namespace
 
-extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
+namespace {
+int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
     SVDQ_REQUIRE(a, "gemm: null args");
     SVDQ_REQUIRE(a->act && a->ascales && a->wgt && a->wscales, "gemm: act/ascales/wgt/wscales must not be null");
     SVDQ_REQUIRE(!a->fp4 || a->colnorm, "gemm: NVFP4 needs colnorm");
@@ -282,5 +345,10 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) {
     if (hipGetDevice(&dev) != hipSuccess) return fail(SVDQ_ELAUNCH, "gemm: cannot identify the current device");
     const int ncu = compute_units(dev);
     if (ncu <= 0) return fail(SVDQ_ELAUNCH, "gemm: cannot query the number of compute units");
-    return a->fp4 ? gemm_fp4(a, (hipStream_t)stream, dev, ncu) : gemm_int4(a, (hipStream_t)stream, dev, ncu);
+    return a->fp4 ? gemm_fp4(a, (hipStream_t)stream, dev, ncu, noalloc) : gemm_int4(a, (hipStream_t)stream, dev, ncu, noalloc);
 }
+}  // namespace
+
+extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) { return gemm_entry(a, stream, false); }
+
+extern "C" int svdq_gemm_w4a4_noalloc(const svdq_gemm_args *a, void *stream) { return gemm_entry(a, stream, true); }

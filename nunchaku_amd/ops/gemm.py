@@ -17,6 +17,9 @@ NORM_EPS = 1e-6  # gemm_w4a4_launch_impl.cuh:374
 # Tuning / testing knob handed to the C ABI as ``k_split``: None lets the library decide, n > 0 splits
 # every output tile along K into n parts (1: never split).  No counterpart in the reference.
 K_SPLIT: int | None = None
+# True routes the call to ``svdq_gemm_w4a4_noalloc`` of the C ABI (same kernels, workspace from a fixed array
+# in device memory instead of an allocation; for callers that cannot allocate, e.g. under graph capture).
+NO_ALLOC: bool = False
 
 
 def _expect(name: str, t: torch.Tensor | None, shape: tuple, dtype: torch.dtype | None, dev: torch.device) -> None:
@@ -180,7 +183,8 @@ def svdq_gemm_w4a4(
         rot_rows=0 if rot_n is None else rot_n.shape[0], norm_eps=NORM_EPS, k_split=int(K_SPLIT or 0),
     )
     with torch.cuda.device(dev):  # the library launches on the current device
-        nv.check(nv.lib().svdq_gemm_w4a4(ctypes.byref(args), nv.stream_ptr(dev)))
+        entry = nv.lib().svdq_gemm_w4a4_noalloc if NO_ALLOC else nv.lib().svdq_gemm_w4a4
+        nv.check(entry(ctypes.byref(args), nv.stream_ptr(dev)))
 
 
 svdq_gemm_w4a4_cuda = svdq_gemm_w4a4
