@@ -19,17 +19,22 @@ def test_constants():
 
 
 def test_int4_known_answers():
-    # one group whose absmax is 7 -> s = fl32(7 * fl32(1/7)); hand-evaluated codes
+    # one group whose absmax is 7: 7 * fl32(1/7) = 1.0000000447 rounds to 1.0 in fp32, so s = 1, r = 1 and
+    # the codes are the inputs rounded half to even (worked out by hand, literal)
     x = torch.zeros(1, 64)
     x[0, :8] = torch.tensor([7.0, -7.0, 3.5, 2.5, 1.5, 0.5, -0.5, -3.5])
     codes, scales = quant.quantize_act_int4(x.to(torch.bfloat16))
-    s32 = np.float32(7.0) * quant.RECIP_7
     assert scales.shape == (1, 1)
-    assert float(scales[0, 0]) == float(torch.tensor(float(s32)).to(torch.bfloat16))
-    r = np.float32(1.0) / s32
-    want = [int(np.rint(np.float32(v) * r)) for v in [7.0, -7.0, 3.5, 2.5, 1.5, 0.5, -0.5, -3.5]]
-    assert codes[0, :8].tolist() == want
+    assert scales[0, 0].view(torch.int16).item() == 0x3F80  # bf16 1.0
+    assert codes[0, :8].tolist() == [7, -7, 4, 2, 2, 0, 0, -4]
     assert codes[0, 8:].abs().max() == 0
+    # absmax 3 -> s = 3 * fl32(1/7) = 0.42857146 (stored bf16 0x3EDB = 0.427734375), r = 2.3333333:
+    # 1 -> 2.33 -> 2, 2 -> 4.67 -> 5, -0.75 -> -1.75 -> -2
+    x2 = torch.zeros(1, 64)
+    x2[0, :4] = torch.tensor([3.0, 1.0, 2.0, -0.75])
+    codes2, scales2 = quant.quantize_act_int4(x2.to(torch.bfloat16))
+    assert scales2[0, 0].view(torch.int16).item() == 0x3EDB
+    assert codes2[0, :4].tolist() == [7, 2, 5, -2]
 
 
 def test_int4_ties_round_half_even():
@@ -37,11 +42,9 @@ def test_int4_ties_round_half_even():
     x = torch.zeros(1, 64)
     x[0, :5] = torch.tensor([14.0, 1.0, 3.0, 5.0, -5.0])
     codes, scales = quant.quantize_act_int4(x.to(torch.bfloat16))
-    s32 = np.float32(14.0) * quant.RECIP_7
-    r = np.float32(1.0) / s32
-    for v, c in zip([1.0, 3.0, 5.0, -5.0], codes[0, 1:5].tolist()):
-        assert c == int(np.rint(np.float32(v) * r))
-    assert codes[0, 0] == 7
+    # 14 * fl32(1/7) = 2.00000009 rounds to 2.0: r = 0.5 and 0.5, 1.5, 2.5, -2.5 are exact ties -> 0, 2, 2, -2
+    assert scales[0, 0].view(torch.int16).item() == 0x4000
+    assert codes[0, :5].tolist() == [7, 0, 2, 2, -2]
 
 
 def test_int4_unsigned_shift_and_clamp():
@@ -52,9 +55,11 @@ def test_int4_unsigned_shift_and_clamp():
     assert codes.min() >= 0 and codes.max() <= 15
     assert codes[0, 1:].max() == 0  # negative inputs clamp to 0
     assert codes[0, 0] == 15
-    # scale uses 1/15 of the shifted absmax
-    amax = float((torch.tensor(15.0) + quant.SHIFT_GELU).to(torch.bfloat16))
-    assert float(scales[0, 0]) == float(torch.tensor(float(np.float32(amax) * quant.RECIP_15)).to(torch.bfloat16))
+    # scale uses 1/15 of the shifted absmax: bf16(15 + 0.171875) = 15.1875, times fl32(1/15) = 1.0125,
+    # stored bf16 1.015625 (0x3F82)
+    assert scales[0, 0].view(torch.int16).item() == 0x3F82
+    # row 1: -1 + 0.171875 < 0 nowhere (linspace 0..3): largest shifted value bf16(3.171875) = 3.171875 -> code 15
+    assert codes[1, 63] == 15 and codes[1, 0] == 1  # 0.171875 / (3.171875 / 15) = 0.81 -> 1
 
 
 def test_int4_zero_group_and_invariants():
@@ -118,12 +123,11 @@ def test_nvfp4_known_answers():
     x[0, 16] = 4000.0  # scale saturates at 448
     codes, scales = quant.quantize_act_nvfp4(x.to(torch.bfloat16))
     assert scales.dtype == torch.float8_e4m3fn and scales.shape == (2, 1)
-    s0 = np.float32(6.0) * quant.RECIP_6
-    assert float(scales[0, 0].float()) == float(torch.tensor(float(s0)).to(torch.float8_e4m3fn).float())
-    r0 = np.float32(1.0) / s0
-    want = quant.e2m1_encode(torch.tensor([float(np.float32(v) * r0) for v in [6.0, 3.0, -1.5, 0.5]])).tolist()
-    assert codes[0, :4].tolist() == want
-    assert float(scales[1, 0].float()) == 448.0
+    # 6 * fl32(1/6) = 1.00000003 rounds to 1.0: scale e4m3 1.0 (0x38), codes are the E2M1 patterns of the inputs:
+    # 6 -> 7, 3 -> 5, -1.5 -> sign | 3 = 11, 0.5 -> 1
+    assert scales[0, 0].view(torch.uint8).item() == 0x38
+    assert codes[0, :4].tolist() == [7, 5, 11, 1]
+    assert scales[1, 0].view(torch.uint8).item() == 0x7E and float(scales[1, 0].float()) == 448.0
     assert codes[0, 16] == 7  # 4000/448 saturates to 6
     assert (codes[0, 17:] == 0).all()
 
