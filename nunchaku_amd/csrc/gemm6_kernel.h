@@ -139,11 +139,18 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     const uint32_t stride_x = low ? 4 * FRAG_BYTES : 2048, stride_q = (uint32_t)p.M_pad * 2;
     const uint32_t dst_w = lds_base + ST_W + wave * 3072, dst_a = lds_base + ST_A + wave * 1024;
     const uint32_t dst_x = lds_base + (low ? ST_A + (4 + wave) * 1024 : ST_WS + (wave - 2) * 1024), dst_q = lds_base + ST_AS;
-    auto issue_copies = [&](uint32_t stage_off) {  // the next k-group not yet requested, into the stage at stage_off
+    // (in three parts, so that the main loop can spread them over its steps: a wave that issues its six
+    // requests back to back stands still until the memory pipeline has taken them, about 30 cycles each)
+    auto issue_copies_a = [&](uint32_t stage_off) {  // the next k-group not yet requested, into the stage at stage_off
         asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\t"
-                     "global_load_lds_dwordx4 %2, %3\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024\n\tglobal_load_lds_dwordx4 %2, %3 offset:2048"
+                     "global_load_lds_dwordx4 %2, %3\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024"
                      :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+    };
+    auto issue_copies_b = [&](uint32_t stage_off) {
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:2048" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
         asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_a), "s"(stage_off), "v"(copy_voff), "s"(src_a) : "memory");
+    };
+    auto issue_copies_c = [&](uint32_t stage_off) {
         asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_x), "s"(stage_off), "v"(copy_voff), "s"(src_x) : "memory");
         uint32_t voff4;
         asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(voff4) : "v"(copy_voff));
@@ -152,6 +159,11 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         src_a += 4 * FRAG_BYTES;
         src_x += stride_x;
         src_q += stride_q;
+    };
+    auto issue_copies = [&](uint32_t stage_off) {
+        issue_copies_a(stage_off);
+        issue_copies_b(stage_off);
+        issue_copies_c(stage_off);
     };
 
     // what the upper half-wave reads as its activation scale
@@ -241,7 +253,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         // stage, whose copies every wave has waited for, may be read.
         if (BULK) {
             asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            issue_copies(sb);  // group l + 3 into the stage of group l
+            issue_copies_a(sb);  // group l + 3 into the stage of group l, two requests per step
         } else {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
@@ -249,7 +261,9 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         read_w(sb_next, 0, W[0], wsop[0]);
         SVDQ_FMA(5, 1)
         __builtin_amdgcn_sched_barrier(0);
+        if (BULK) issue_copies_b(sb);
         SVDQ_STEP(6, 0, 1, W[1], X[1], wsop[1], asop[1], 3, read_x(sb_next, 1, X[1], asop[1]))
+        if (BULK) issue_copies_c(sb);
         // (tile 0 of the next group; of nothing after the last group)
         SVDQ_STEP(7, 1, 0, W[0], X[0], wsop[0], asop[0], 0, )
         sb = sb_next;
