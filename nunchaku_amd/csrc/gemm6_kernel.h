@@ -139,39 +139,42 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     const uint32_t stride_x = low ? 4 * FRAG_BYTES : 2048, stride_q = (uint32_t)p.M_pad * 2;
     const uint32_t dst_w = lds_base + ST_W + wave * 3072, dst_a = lds_base + ST_A + wave * 1024;
     const uint32_t dst_x = lds_base + (low ? ST_A + (4 + wave) * 1024 : ST_WS + (wave - 2) * 1024), dst_q = lds_base + ST_AS;
-    // (in three parts, so that the main loop can spread them over its steps: a wave that issues its six
-    // requests back to back stands still until the memory pipeline has taken them, about 30 cycles each)
-    auto issue_copies_a = [&](uint32_t stage_off) {  // the next k-group not yet requested, into the stage at stage_off
-        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\t"
-                     "global_load_lds_dwordx4 %2, %3\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024"
-                     :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+    // The requests of a k-group are issued one at a time, spread over the steps of the main loop: a wave
+    // that issues its six requests back to back stands still until the memory pipeline has taken them,
+    // about 30 cycles each.  First the three weight chunks (W), later the other three (R).
+    auto copy_w = [&](uint32_t stage_off, int i) {  // weight chunk i of the next k-group whose weights are not requested yet
+        if (i == 0) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+        if (i == 1) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+        if (i == 2) {
+            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:2048" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+            src_w += 8 * FRAG_BYTES;
+        }
     };
-    auto issue_copies_b = [&](uint32_t stage_off) {
-        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:2048" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
-        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_a), "s"(stage_off), "v"(copy_voff), "s"(src_a) : "memory");
-    };
-    auto issue_copies_c = [&](uint32_t stage_off) {
-        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_x), "s"(stage_off), "v"(copy_voff), "s"(src_x) : "memory");
-        uint32_t voff4;
-        asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(voff4) : "v"(copy_voff));
-        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3" :: "s"(dst_q), "s"(stage_off), "v"(voff4), "s"(src_q) : "memory");
-        src_w += 8 * FRAG_BYTES;
-        src_a += 4 * FRAG_BYTES;
-        src_x += stride_x;
-        src_q += stride_q;
-    };
-    auto issue_copies = [&](uint32_t stage_off) {
-        issue_copies_a(stage_off);
-        issue_copies_b(stage_off);
-        issue_copies_c(stage_off);
+    auto copy_r = [&](uint32_t stage_off, int i) {  // the rest: activation chunk, activation / weight-scale chunk, activation scales
+        if (i == 0) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_a), "s"(stage_off), "v"(copy_voff), "s"(src_a) : "memory");
+        if (i == 1) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_x), "s"(stage_off), "v"(copy_voff), "s"(src_x) : "memory");
+        if (i == 2) {
+            uint32_t voff4;
+            asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(voff4) : "v"(copy_voff));
+            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3" :: "s"(dst_q), "s"(stage_off), "v"(voff4), "s"(src_q) : "memory");
+            src_a += 4 * FRAG_BYTES;
+            src_x += stride_x;
+            src_q += stride_q;
+        }
     };
 
     // what the upper half-wave reads as its activation scale
     if (tid < STAGES * 32) *(uint32_t *)(lds + (tid >> 5) * STAGE_BYTES + ST_Z + (tid & 31) * 4) = 0u;
 
-    issue_copies(0);
-    if (ng > 1) issue_copies(STAGE_BYTES);
-    if (ng > 2) issue_copies(2 * STAGE_BYTES);
+    // groups 0 and 1 entirely, the weights of group 2
+    for (int i = 0; i < 3; i++) copy_w(0, i);
+    for (int i = 0; i < 3; i++) copy_r(0, i);
+    if (ng > 1) {
+        for (int i = 0; i < 3; i++) copy_w(STAGE_BYTES, i);
+        for (int i = 0; i < 3; i++) copy_r(STAGE_BYTES, i);
+    }
+    if (ng > 2)
+        for (int i = 0; i < 3; i++) copy_w(2 * STAGE_BYTES, i);
 
     // per-lane read offsets inside a stage
     const uint32_t off16 = lane * 16, off8 = 1024 + lane * 8;
@@ -197,7 +200,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         for (int e = 0; e < 16; e++) acc[t][e] = 0.f;
 
     // group 0 has landed
-    if (ng > 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    if (ng > 2) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     else if (ng > 1) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -233,15 +236,22 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
 
     uint32_t sb = 0;  // byte offset of the stage of group l
     // The loop body is one basic block (a branch inside it lets the compiler sink the fma of all steps
-    // below the branch, with all their operands alive).  BULK: the groups that still have copies to
-    // request (l + 3 < ng); the last three groups run the same body without requests and wait for
-    // everything outstanding.
-    auto group_body = [&](auto BULK_T) {
-        constexpr bool BULK = decltype(BULK_T)::value;
+    // below the branch, with all their operands alive).  Requests of iteration l: in steps 0-2 the rest of
+    // group l + 2 (its stage, that of group l - 1, was free since the previous barrier and already
+    // received the weights), in steps 5-7, behind the barrier, the weights of group l + 3 into the stage
+    // of group l.  At the barrier group l + 1 must have landed; the six requests of group l + 2 are the
+    // only ones issued after it.  MODE 2: both (l + 3 < ng), 1: only the rest of group l + 2 (l = ng - 3),
+    // 0: nothing left to request.
+    auto group_body = [&](auto MODE_T) {
+        constexpr int MODE = decltype(MODE_T)::value;
         const uint32_t sb_next = sb == (STAGES - 1) * STAGE_BYTES ? 0 : sb + STAGE_BYTES;
+        const uint32_t sb_prev = sb == 0 ? (STAGES - 1) * STAGE_BYTES : sb - STAGE_BYTES;
         // step t issues the matrix instructions of tile t + 1 (tile = 2 nt + mt) and accumulates tile t
+        if (MODE >= 1) copy_r(sb_prev, 0);
         SVDQ_STEP(0, 0, 1, W[0], X[1], wsop[0], asop[1], 3, read_w(sb, 1, W[1], wsop[1]))
+        if (MODE >= 1) copy_r(sb_prev, 1);
         SVDQ_STEP(1, 1, 0, W[1], X[0], wsop[1], asop[0], 0, )
+        if (MODE >= 1) copy_r(sb_prev, 2);
         SVDQ_STEP(2, 0, 1, W[1], X[1], wsop[1], asop[1], 3, read_w(sb, 2, W[0], wsop[0]))
         SVDQ_STEP(3, 1, 0, W[0], X[0], wsop[0], asop[0], 0, )
         SVDQ_STEP(4, 0, 1, W[0], X[1], wsop[0], asop[1], 3, read_w(sb, 3, W[1], wsop[1]))
@@ -251,26 +261,27 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         // Every LDS read of this group has been issued, and the last one has arrived (the instruction
         // above needed it).  Behind the barrier the stage may be overwritten, and the next group's
         // stage, whose copies every wave has waited for, may be read.
-        if (BULK) {
-            asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            issue_copies_a(sb);  // group l + 3 into the stage of group l, two requests per step
-        } else {
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        }
+        if (MODE >= 1) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (MODE == 2) copy_w(sb, 0);
         read_x(sb_next, 0, X[0], asop[0]);
         read_w(sb_next, 0, W[0], wsop[0]);
         SVDQ_FMA(5, 1)
         __builtin_amdgcn_sched_barrier(0);
-        if (BULK) issue_copies_b(sb);
+        if (MODE == 2) copy_w(sb, 1);
         SVDQ_STEP(6, 0, 1, W[1], X[1], wsop[1], asop[1], 3, read_x(sb_next, 1, X[1], asop[1]))
-        if (BULK) issue_copies_c(sb);
+        if (MODE == 2) copy_w(sb, 2);
         // (tile 0 of the next group; of nothing after the last group)
         SVDQ_STEP(7, 1, 0, W[0], X[0], wsop[0], asop[0], 0, )
         sb = sb_next;
     };
     int l = 0;
-    for (; l + 3 < ng; l++) group_body(std::true_type{});
-    for (; l < ng; l++) group_body(std::false_type{});
+    for (; l + 3 < ng; l++) group_body(std::integral_constant<int, 2>{});
+    if (l + 2 < ng) {
+        group_body(std::integral_constant<int, 1>{});
+        l++;
+    }
+    for (; l < ng; l++) group_body(std::integral_constant<int, 0>{});
 #undef SVDQ_STEP
 #undef SVDQ_FMA
     __syncthreads();  // the ring is free: the epilogue reuses it
