@@ -66,6 +66,8 @@ class SVDQW4A4Linear(nn.Module):
             self.wcscales = nn.Parameter(torch.ones(out_features, dtype=torch_dtype, device=device), requires_grad=False)
 
         self.act_unsigned = act_unsigned
+        # one factor per 16 ranks of the low-rank branch (src/Linear.h:98); None: all ones
+        self.lora_scales: list[float] | None = None
         self._native: dict[str, torch.Tensor | None] | None = None
         self._native_stamp: tuple | None = None
         self._alpha: float | None = None
@@ -130,6 +132,31 @@ class SVDQW4A4Linear(nn.Module):
             }
         return self._native
 
+    # ---- low-rank hot swap ---------------------------------------------------------------------
+    def update_lora(self, proj_down: torch.Tensor, proj_up: torch.Tensor) -> None:
+        """Replace the low-rank branch by ``proj_down`` [K, R'] / ``proj_up`` [N, R'] (reference packed order,
+        e.g. the layer's own branch with a user LoRA's ranks appended, ``checkpoint.concat_lowrank``).  The
+        rank may change; the per-16-rank factors start again at one (GEMM_W4A4::loadParam,
+        src/Linear.cpp:124-134)."""
+        if proj_down.shape[0] != self.in_features or proj_up.shape[0] != self.out_features or proj_down.shape[1] != proj_up.shape[1]:
+            raise ValueError(f"expected proj_down [{self.in_features}, R] and proj_up [{self.out_features}, R], got {tuple(proj_down.shape)} and {tuple(proj_up.shape)}")
+        if proj_down.shape[1] % 16 != 0 or proj_down.shape[1] > 128:
+            raise ValueError("the rank must be a multiple of 16, at most 128")
+        dev, dt = self.proj_down.device, self.proj_down.dtype
+        self.proj_down = nn.Parameter(proj_down.detach().to(device=dev, dtype=dt).contiguous(), requires_grad=False)
+        self.proj_up = nn.Parameter(proj_up.detach().to(device=dev, dtype=dt).contiguous(), requires_grad=False)
+        self.rank = proj_down.shape[1]
+        self.lora_scales = None
+        self.invalidate_native()
+
+    def set_lora_scale(self, skip_ranks: int, scale: float) -> None:
+        """Factor ``scale`` on every rank behind the first ``skip_ranks`` (the layer's own branch keeps 1):
+        QuantizedFluxModel::setLoraScale, nunchaku/csrc/flux.h:177-196."""
+        if skip_ranks % 16 != 0:
+            raise ValueError("skip_ranks must be a multiple of 16")
+        groups = (self.rank + 15) // 16
+        self.lora_scales = [1.0 if i < skip_ranks // 16 else float(scale) for i in range(groups)]
+
     @property
     def alpha(self) -> float:
         """Per-tensor weight scale as a host float, read once (the reference hands the parameter to a
@@ -168,7 +195,7 @@ class SVDQW4A4Linear(nn.Module):
         svdq_gemm_w4a4(
             act=quantized_x, wgt=t["qweight"], out=output, ascales=ascales, wscales=t["wscales"],
             lora_act_in=lora_act, lora_up=t["proj_up"], bias=t["bias"], fp4=self.precision == "nvfp4",
-            alpha=self.alpha, wcscales=t["wcscales"], act_unsigned=self.act_unsigned,
+            alpha=self.alpha, wcscales=t["wcscales"], act_unsigned=self.act_unsigned, lora_scales=self.lora_scales,
         )
         return output
 

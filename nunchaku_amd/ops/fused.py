@@ -29,7 +29,7 @@ def fused_gelu_mlp(x: torch.Tensor, fc1, fc2, pad_size: int = 256) -> torch.Tens
         act=quantized_x, wgt=t1["qweight"], qout=qout_act, ascales=ascales, wscales=t1["wscales"],
         oscales=qout_ascales, lora_act_in=lora_act, lora_up=t1["proj_up"], lora_down=t2["proj_down"],
         lora_act_out=qout_lora_act, bias=t1["bias"], smooth_factor=t2["smooth_factor"],
-        fp4=fc1.precision == "nvfp4", alpha=fc1.alpha, wcscales=t1["wcscales"],
+        fp4=fc1.precision == "nvfp4", alpha=fc1.alpha, wcscales=t1["wcscales"], lora_scales=fc1.lora_scales,
     )
     output = torch.empty(batch_size * seq_len, fc2.out_features, dtype=x.dtype, device=x.device)
     output = fc2.forward_quant(qout_act, qout_ascales, qout_lora_act, output=output)
@@ -53,6 +53,7 @@ def fused_qkv_norm_rottary(x: torch.Tensor, proj, norm_q, norm_k, rotary_emb: to
         act=quantized_x, wgt=t["qweight"], out=output, ascales=ascales, wscales=t["wscales"],
         lora_act_in=lora_act, lora_up=t["proj_up"], bias=t["bias"], fp4=proj.precision == "nvfp4",
         alpha=proj.alpha, wcscales=t["wcscales"], norm_q=norm_q.weight, norm_k=norm_k.weight, rotary_emb=rotary_emb,
+        lora_scales=proj.lora_scales,
     )
     # (the reference views the padded buffer directly, which only works for token counts that need no padding)
     return output[: batch_size * seq_len].view(batch_size, seq_len, -1)

@@ -97,3 +97,46 @@ CONFIGS = {
     "c4_out": dict(M=4608, K=15360, N=3072, R=32, seed=3, fp4=True),
     "c5": dict(M=18432, K=3072, N=12288, R=128, seed=4),
 }
+
+
+# ---------------------------------------------------------------------------------------------
+# A small checkpoint with the reference's key names, for the ingestion tests.
+# ---------------------------------------------------------------------------------------------
+
+# (checkpoint module name inside a block, N, K) of a toy double-stream block and a toy single-stream block;
+# the names are those a reference checkpoint holds BEFORE convert_flux_state_dict
+# (nunchaku/models/transformers/transformer_flux_v2.py:395-450)
+TOY_BLOCK_LAYERS = {
+    "transformer_blocks.0": (("qkv_proj", 384, 128), ("qkv_proj_context", 384, 128), ("out_proj", 128, 128), ("out_proj_context", 128, 128),
+                             ("mlp_fc1", 256, 128), ("mlp_fc2", 128, 256), ("mlp_context_fc1", 256, 128), ("mlp_context_fc2", 128, 256)),
+    "single_transformer_blocks.0": (("qkv_proj", 384, 128), ("mlp_fc1", 256, 128), ("mlp_fc2", 128, 256), ("out_proj", 128, 128)),
+}
+
+
+def toy_checkpoint(rank: int = 16, fp4_blocks: tuple[str, ...] = ()) -> tuple[dict[str, torch.Tensor], dict[str, LogicalLayer]]:
+    """State dict in the reference's checkpoint naming (``lora_down``, ``lora_up``, ``smooth``,
+    ``smooth_orig``, block-local module names) and the logical layers it was made from, keyed by the
+    checkpoint prefix.  NVFP4 layers come without ``wtscale`` / ``wcscales`` when their seed is even, as
+    older checkpoints do."""
+    sd: dict[str, torch.Tensor] = {}
+    layers: dict[str, LogicalLayer] = {}
+    seed = 100
+    for block, specs in TOY_BLOCK_LAYERS.items():
+        for name, n, k in specs:
+            seed += 1
+            fp4 = block in fp4_blocks
+            layer = make_layer(n, k, rank, seed=seed, fp4=fp4, bias=name != "mlp_fc2")
+            if fp4 and seed % 2 == 0:
+                layer.wtscale = 1.0
+            ref = to_reference_checkpoint(layer)
+            prefix = f"{block}.{name}"
+            for key, value in ref.items():
+                ck = {"proj_down": "lora_down", "proj_up": "lora_up", "smooth_factor": "smooth", "smooth_factor_orig": "smooth_orig"}.get(key, key)
+                if fp4 and seed % 2 == 0 and key in ("wtscale", "wcscales"):
+                    continue
+                sd[f"{prefix}.{ck}"] = value
+            layers[prefix] = layer
+        sd[f"{block}.norm_q.weight"] = torch.ones(128, dtype=torch.bfloat16)
+        sd[f"{block}.norm_k.weight"] = torch.ones(128, dtype=torch.bfloat16)
+    sd["x_embedder.weight"] = torch.zeros(4, 4, dtype=torch.bfloat16)  # an unquantized tensor passes through
+    return sd, layers
