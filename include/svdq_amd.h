@@ -106,7 +106,9 @@ typedef struct svdq_quantize_args {
     const float *smooth_rcp;/* fp32 [K] from svdq_repack_smooth, or NULL for no smoothing          */
     int64_t M, M_pad, K, R;
     int32_t fp4;            /* 0: INT4 group 64 (signed); 1: NVFP4 group 16                        */
-    int32_t fuse_glu;       /* must be 0 (not implemented)                                         */
+    int32_t fuse_glu;       /* 1: input is bf16 [M, 2K], pairs (value, gate); the K columns that are
+                               quantized and projected are bf16(value * bf16(gate * sigmoid(gate)))
+                               (load_act_to_fpsum<fuse_glu>, gemm_base.cuh:612-623)                */
 } svdq_quantize_args;
 
 int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *stream);

@@ -29,7 +29,7 @@ using namespace svdq;
 namespace {
 
 struct QuantParams {
-    const uint16_t *x;       // bf16 [M, K]
+    const uint16_t *x;       // bf16 [M, K], or [M, 2K] (value, gate) pairs when the kernel applies the gated unit
     uint8_t *act;            // INT4: E2M3 fragments [M_pad/128][K/64][4]; NVFP4: nibble tiles [M_pad/32][K/64][32][32 B]
     void *oscales;           // bf16 [K/64, M_pad] or fp8 [K/16, M_pad]
     const bf16x8_t *down;    // native proj_down
@@ -42,7 +42,12 @@ constexpr uint32_t RSRC_WORD3 = 0x00020000;  // raw buffer, 32-bit data format
 
 // SMOOTH: 0 = no smoothing factors, 1 = the K reciprocal factors are copied to LDS once per workgroup,
 // 2 = read from global memory per chunk (K too large for LDS).
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH>
+//
+// GLU: the input row holds 2K columns, pairs (value, gate); the K columns that are smoothed, quantized
+// and projected are bf16(value * bf16(gate * sigmoid(gate))) (load_act_to_fpsum<fuse_glu>,
+// gemm_base.cuh:612-623; silu, gemm_utils.cuh:322-327).  A lane then reads 64 consecutive input columns
+// for its 32, and everything after the product is as without GLU.
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU>
 __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams p) {
     extern __shared__ float lds[];  // smoothing factors [K] during the walk, then [NW waves][MT][RT][64][4] partial projections
     const int lane = threadIdx.x & 63;
@@ -65,25 +70,28 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
     rows_valid = rows_valid < 0 ? 0 : (rows_valid > 16 * MT ? 16 * MT : rows_valid);
     // (descriptor words made scalar explicitly: a descriptor the compiler takes for lane-dependent is
     // looped over lane by lane)
-    const uint64_t xbase = (uint64_t)(p.x + (size_t)row0 * p.K);
+    constexpr int XW = GLU ? 2 : 1;  // input columns per quantized column
+    constexpr int XL = 4 * XW;       // 16-byte loads per lane, tile and chunk
+    const int ld = XW * p.K;         // input row length
+    const uint64_t xbase = (uint64_t)(p.x + (size_t)row0 * ld);
     const uint64_t xbase_s = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(xbase >> 32)) << 32) |
                              (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)xbase);
     const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void *)xbase_s, 0, __builtin_amdgcn_readfirstlane(rows_valid * p.K * 2), RSRC_WORD3);
-    const uint32_t x_voff = (uint32_t)(r * p.K + 32 * q) * 2;
+        __builtin_amdgcn_make_buffer_rsrc((void *)xbase_s, 0, __builtin_amdgcn_readfirstlane(rows_valid * ld * 2), RSRC_WORD3);
+    const uint32_t x_voff = (uint32_t)(r * ld + 32 * XW * q) * 2;
 
-    // x of one chunk: MT tiles x 4 steps x 8 bf16 per lane
+    // x of one chunk: MT tiles x 4 steps x 8 bf16 per lane (twice that with GLU)
     // Requests are unconditional (a request behind a branch makes the compiler's wait counting assume the
     // worst on every path and wait for the chunks requested ahead): a chunk index past the end gets a lane
     // offset beyond the buffer size instead, which reads zeros and touches no memory.  (The hardware checks
     // the lane offset against the size, not the scalar offset that carries the chunk.)
-    auto load_x = [&](int c, u32x4_t (&xv)[MT][4]) {
+    auto load_x = [&](int c, u32x4_t (&xv)[MT][XL]) {
         const uint32_t beyond = c < nchunks ? 0u : 0x80000000u;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                xv[mt][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (x_voff | beyond) + (uint32_t)(16 * mt * p.K) * 2 + 16 * i, c * 256, 0);
+            for (int i = 0; i < XL; i++)
+                xv[mt][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (x_voff | beyond) + (uint32_t)(16 * mt * ld) * 2 + 16 * i, c * 256 * XW, 0);
     };
     // proj_down as a buffer too: empty when there is no low-rank branch, so that its requests need no branch
     const __amdgpu_buffer_rsrc_t drsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.down, 0, RT > 0 ? p.K * p.R * 2 : 0, RSRC_WORD3);
@@ -92,7 +100,7 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
     };
 
     // DEPTH chunks are requested ahead of the one being worked on
-    u32x4_t xv[DEPTH + 1][MT][4];
+    u32x4_t xv[DEPTH + 1][MT][XL];
 #pragma unroll
     for (int s = 0; s < DEPTH; s++) load_x(wave + s * NW, xv[s]);
 
@@ -101,7 +109,7 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
         __syncthreads();
     }
 
-    auto process = [&](int c, u32x4_t (&x)[MT][4], u32x4_t (&x_ahead)[MT][4]) {
+    auto process = [&](int c, u32x4_t (&xraw)[MT][XL], u32x4_t (&x_ahead)[MT][XL]) {
         const int kbase = 128 * c + 32 * q;
         // ---- requests first: the low-rank operands of this chunk (all four steps when they fit the
         // registers), then the activations DEPTH chunks ahead.  In this order a wait for the operands
@@ -116,6 +124,31 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
         }
         load_x(c + DEPTH * NW, x_ahead);
         __builtin_amdgcn_sched_barrier(0);
+
+        // ---- the gated unit: 16 (value, gate) pairs of two loads become the 8 bf16 of one step
+        u32x4_t xglu[GLU ? MT : 1][4];
+        if (GLU) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float v[2];
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            const uint32_t w = xraw[mt][2 * i + (2 * j + h) / 4][(2 * j + h) % 4];
+                            const float val = bits_f32(w << 16), gate = bits_f32(w & 0xFFFF0000u);
+                            const float sg = gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gate));
+                            v[h] = val * bits_f32(f32_to_bf16_bits(sg) << 16);
+                        }
+                        xglu[mt][i][j] = pack_bf16x2(v[0], v[1]);
+                    }
+        }
+        auto xs = [&](int mt, int i) -> u32x4_t {
+            if constexpr (GLU) return xglu[mt][i];
+            else return xraw[mt][i];
+        };
 
         // ---- smooth, quantize, store
 #pragma unroll
@@ -134,8 +167,14 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
                 }
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const uint32_t w = x[mt][i][j];
-                    const float lo = bits_f32(w << 16), hi = bits_f32(w & 0xFFFF0000u);
+                    const uint32_t w = xs(mt, i)[j];
+                    float lo = bits_f32(w << 16), hi = bits_f32(w & 0xFFFF0000u);
+                    if (FP4) {
+                        // the reference adds its shift (zero here) before the division, which turns -0 into
+                        // +0 (gemm_w4a4.cuh:986); only the E2M1 sign bit can tell the difference
+                        lo += 0.0f;
+                        hi += 0.0f;
+                    }
                     const int e = 8 * i + 2 * j;
                     if (SMOOTH) {
                         // bf16(x / smooth) for the pair: two products, one packed hardware rounding
@@ -183,7 +222,7 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
                 const bf16x8_t b = DOWN_UPFRONT ? dn[i][rt] : load_down(c, i, rt);
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++)
-                    acc[mt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, x[mt][i]), b, acc[mt][rt], 0, 0, 0);
+                    acc[mt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xs(mt, i)), b, acc[mt][rt], 0, 0, 0);
             }
     };
 
@@ -222,11 +261,11 @@ walked:
 
 constexpr size_t SMOOTH_LDS_MAX = 64 * 1024;  // two workgroups of a compute unit must fit side by side
 
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU>
 int launch_as(const QuantParams &p, hipStream_t stream) {
     size_t smem = (size_t)NW * MT * (p.R / 16) * 64 * 4 * sizeof(float);
     if (SMOOTH == 1 && (size_t)p.K * 4 > smem) smem = (size_t)p.K * 4;
-    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH>;
+    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH, GLU>;
     if (smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "quantize: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
@@ -235,22 +274,29 @@ int launch_as(const QuantParams &p, hipStream_t stream) {
     return check_launch("quantize_w4a4_act_fuse_lora");
 }
 
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, bool GLU>
 int launch(const QuantParams &p, hipStream_t stream) {
-    if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0>(p, stream);
-    if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1>(p, stream);
-    return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2>(p, stream);
+    if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0, GLU>(p, stream);
+    if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1, GLU>(p, stream);
+    return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2, GLU>(p, stream);
 }
 
-template <bool FP4>
+template <bool FP4, bool GLU>
 int dispatch(const QuantParams &p, hipStream_t stream) {
     // Rows per workgroup: 16 while that gives the chip enough workgroups, 32 to amortise the proj_down
     // reads at high rank.  Four waves of up to 256 registers: two workgroups fit a compute unit, so that a
     // workgroup count a little above the number of compute units does not cost a second round.
     const int RT = p.R / 16;
-    if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4>(p, stream) : launch<4, 1, 2, 2, FP4>(p, stream);
-    if (RT <= 4) return launch<4, 2, 4, 1, FP4>(p, stream);
-    if (RT <= 8) return launch<4, 2, 8, 1, FP4>(p, stream);
+    // (with GLU a chunk in flight is twice the registers: one chunk ahead, 16 rows)
+    if (GLU) {
+        if (RT <= 2) return launch<4, 1, 2, 1, FP4, true>(p, stream);
+        if (RT <= 4) return launch<4, 1, 4, 1, FP4, true>(p, stream);
+        if (RT <= 8) return launch<4, 1, 8, 1, FP4, true>(p, stream);
+    } else {
+        if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4, false>(p, stream) : launch<4, 1, 2, 2, FP4, false>(p, stream);
+        if (RT <= 4) return launch<4, 2, 4, 1, FP4, false>(p, stream);
+        if (RT <= 8) return launch<4, 2, 8, 1, FP4, false>(p, stream);
+    }
     return fail(SVDQ_EUNSUPPORTED, "quantize: rank %d > 128 is not supported", p.R);
 }
 
@@ -268,7 +314,6 @@ extern "C" int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *a, voi
     SVDQ_REQUIRE(((uintptr_t)a->input % 16 == 0) && ((uintptr_t)a->output % 16 == 0) && ((uintptr_t)a->lora_down % 16 == 0) &&
                      ((uintptr_t)a->smooth_rcp % 16 == 0),
                  "quantize: pointers must be 16-byte aligned");
-    if (a->fuse_glu) return fail(SVDQ_EUNSUPPORTED, "quantize: fuse_glu is not implemented");
     QuantParams p;
     p.x = (const uint16_t *)a->input;
     p.act = (uint8_t *)a->output;
@@ -277,5 +322,7 @@ extern "C" int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *a, voi
     p.lora_out = a->lora_act_out;
     p.smooth_rcp = a->smooth_rcp;
     p.M = (int)a->M; p.M_pad = (int)a->M_pad; p.K = (int)a->K; p.R = (int)a->R;
-    return a->fp4 ? dispatch<true>(p, (hipStream_t)stream) : dispatch<false>(p, (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    if (a->fuse_glu) return a->fp4 ? dispatch<true, true>(p, s) : dispatch<false, true>(p, s);
+    return a->fp4 ? dispatch<true, false>(p, s) : dispatch<false, false>(p, s);
 }

@@ -26,7 +26,8 @@ def svdq_quantize_w4a4_act_fuse_lora(
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Smooth, quantize to 4 bits and project onto the low-rank basis in one pass over ``input``.
 
-    input  bf16 [M, K];  lora_down  proj_down [K, R];  smooth  smooth_factor [K] (both either in the
+    input  bf16 [M, K] (``fuse_glu``: [M, 2K] pairs (value, gate), the K columns value * silu(gate) are what
+    is quantized and projected);  lora_down  proj_down [K, R];  smooth  smooth_factor [K] (both either in the
     reference checkpoint layout, repacked once and cached, or already native, see ``packing``).
     Returns ``(output u8 [M_pad, 3K/4], oscales [K/G, M_pad], lora_act_out fp32 [M_pad, R])`` where
     M_pad rounds M up to ``pad_size`` (256).  ``output`` is private to this operator and the GEMM: INT4
@@ -44,6 +45,12 @@ def svdq_quantize_w4a4_act_fuse_lora(
     if lora_down is None:
         raise ValueError("lora_down is required")  # the reference reads lora_down.shape[1] unconditionally
     batch_size, channels = input.shape
+    if fuse_glu:
+        # the row holds (value, gate) pairs: half as many columns are quantized (the reference sizes its
+        # checks the same way, gemm_w4a4_launch_impl.cuh:466-480, and leaves the allocation to the caller)
+        if channels % 2:
+            raise ValueError("fuse_glu needs an even number of input columns")
+        channels //= 2
     rank = lora_down.shape[1]
     batch_size_pad = ceil_divide(batch_size, pad_size) * pad_size
     dev = input.device

@@ -19,12 +19,21 @@ def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
     return torch.nn.functional.gelu(x.to(torch.float32), approximate="tanh")
 
 
+def glu_input(x: torch.Tensor) -> torch.Tensor:
+    """[M, 2K] pairs (value, gate) -> bf16 [M, K] ``value * silu(gate)``, each of the two operations
+    rounded to bf16 (gemm_base.cuh:612-623, gemm_utils.cuh:322-327)."""
+    value, gate = x[:, 0::2].to(torch.float64), x[:, 1::2].to(torch.float64)
+    silu = (gate * torch.sigmoid(gate)).to(torch.float32).to(torch.bfloat16)
+    return (value * silu.to(torch.float64)).to(torch.float32).to(torch.bfloat16)
+
+
 def quantize_act_fuse_lora(
     x: torch.Tensor,
     proj_down: torch.Tensor,
     smooth: torch.Tensor | None,
     fp4: bool = False,
     pad_size: int = 256,
+    fuse_glu: bool = False,
 ):
     """quantize_w4a4_fuse_lora_kernel (gemm_w4a4.cuh:1097-1184) behind
     svdq_quantize_w4a4_act_fuse_lora_cuda (nunchaku/ops/quantize.py:11-54).
@@ -33,8 +42,14 @@ def quantize_act_fuse_lora(
     Rows M..M_pad are zero-filled by the loader (gemm_base.cuh:591-646) and therefore quantize to
     code 0 / scale 0 / lora 0.  The low-rank projection uses the raw x (no smoothing):
     gemm_w4a4.cuh:1159-1171.
+    ``fuse_glu``: x is [M, 2K], pairs (value, gate); what is smoothed, quantized and projected is
+    ``bf16(value * bf16(gate * sigmoid(gate)))`` (load_act_to_fpsum<fuse_glu>, gemm_base.cuh:612-623:
+    ``raw[j].x * silu(raw[j].y)`` in the activation type; silu rounds to that type itself,
+    gemm_utils.cuh:322-327).
     Returns (codes [M_pad, K], scales [K/G, M_pad], lora_act fp32 [M_pad, R]).
     """
+    if fuse_glu:
+        x = glu_input(x)
     M, K = x.shape
     M_pad = (M + pad_size - 1) // pad_size * pad_size
     xp = torch.zeros(M_pad, K, dtype=torch.bfloat16)

@@ -56,8 +56,10 @@ def test_quantize_rejects_bad_arguments(lib):
     assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
     assert b"aligned" in lib.svdq_last_error()
     a.input = 16
+    a.R = 144
     a.fuse_glu = 1
     assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -2
+    assert b"rank" in lib.svdq_last_error()
 
 
 def test_gemm_rejects_bad_arguments(lib):

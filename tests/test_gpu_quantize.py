@@ -11,16 +11,17 @@ from oracle import quant, synth
 pytestmark = pytest.mark.gpu
 
 
-def _run(dev, x, layer, fp4=False, smooth=True):
+def _run(dev, x, layer, fp4=False, smooth=True, fuse_glu=False):
     from nunchaku_amd import packing
     from nunchaku_amd.ops import svdq_quantize_w4a4_act_fuse_lora
 
     sd = synth.to_reference_checkpoint(layer)
     out, osc, la = svdq_quantize_w4a4_act_fuse_lora(
-        x.to(dev), lora_down=sd["proj_down"].to(dev), smooth=sd["smooth_factor"].to(dev) if smooth else None, fp4=fp4
+        x.to(dev), lora_down=sd["proj_down"].to(dev), smooth=sd["smooth_factor"].to(dev) if smooth else None, fp4=fp4, fuse_glu=fuse_glu
     )
     torch.cuda.synchronize()
-    return packing.act_to_logical(out.cpu(), x.shape[1], fp4=fp4), packing.scales_to_logical(osc.cpu(), fp4), la.cpu()
+    K = x.shape[1] // (2 if fuse_glu else 1)
+    return packing.act_to_logical(out.cpu(), K, fp4=fp4), packing.scales_to_logical(osc.cpu(), fp4), la.cpu()
 
 
 def _check(x, layer, codes, osc, la, fp4=False, smooth=True):
@@ -123,3 +124,81 @@ def test_rejects_bad_shapes(dev):
     x = torch.zeros(16, 192, dtype=torch.bfloat16, device=dev)  # K not a multiple of 128
     with pytest.raises(ValueError):
         svdq_quantize_w4a4_act_fuse_lora(x, lora_down=torch.zeros(192, 16, dtype=torch.bfloat16, device=dev).contiguous())
+
+
+def test_nvfp4_negative_zero_inputs_give_pattern_zero(dev):
+    """-0.0 inputs: the reference adds a zero shift before smoothing (gemm_w4a4.cuh:986), so the E2M1 sign bit
+    must not be set for them."""
+    M, K, R = 64, 256, 16
+    announce("quantize nvfp4 negative zeros")
+    layer = synth.make_layer(128, K, R, seed=13, fp4=True)
+    x = synth.make_activations(M, K, seed=13)
+    x[::3, ::5] = -0.0
+    x[1] = -0.0
+    for smooth in (True, False):
+        codes, osc, la = _run(dev, x, layer, fp4=True, smooth=smooth)
+        _check(x, layer, codes, osc, la, fp4=True, smooth=smooth)
+        assert (codes[1] == 0).all()
+
+
+def _glu_pairs(value, gate):
+    return torch.stack([value, gate], dim=2).reshape(value.shape[0], -1).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("fp4", [False, True])
+@pytest.mark.parametrize("M,K,R", [(256, 256, 32), (70, 640, 16), (300, 1024, 128), (40, 16512, 64)])
+def test_fuse_glu_saturated_gates_bit_exact(dev, M, K, R, fp4):
+    """Gates where sigmoid is 1 or 0 in fp32 whatever its approximation (|gate| >= 32): silu(gate) is the
+    gate itself or minus zero, and the product value * gate has one correct bf16 rounding.  Codes, scales
+    and the projection are then held to the same bar as without the gated unit; a wrong pair order or
+    column mapping changes every group."""
+    announce(f"quantize fuse_glu saturated gates M={M} K={K} R={R} fp4={fp4}")
+    layer = synth.make_layer(128, K, R, seed=M + K, fp4=fp4)
+    g = torch.Generator().manual_seed(M + K)
+    value = synth.make_activations(M, K, seed=M + 3 * K).float() / 32
+    gate = 32.0 + 8 * torch.rand(M, K, generator=g)
+    gate[torch.rand(M, K, generator=g) < 0.1] = -120.0
+    x2 = _glu_pairs(value, gate)
+    assert x2.shape == (M, 2 * K)
+    codes, osc, la = _run(dev, x2, layer, fp4=fp4, fuse_glu=True)
+    x = olin.glu_input(x2)
+    assert torch.equal(x.float(), (x2[:, 0::2].float() * torch.where(x2[:, 1::2].float() > 0, x2[:, 1::2].float(), torch.zeros(())))
+                       .to(torch.bfloat16).float()), "the oracle itself: silu is the identity or zero here"
+    _check(x, layer, codes, osc, la, fp4=fp4)
+
+
+@pytest.mark.parametrize("fp4", [False, True])
+def test_fuse_glu_random_gates(dev, fp4):
+    """Ordinary gates: sigmoid comes from the hardware's exp2 and reciprocal, the oracle's from libm, so
+    bf16(silu) may differ by one ulp where the fp32 value lies next to a rounding midpoint (a few elements
+    in 10^4 distinct gate values, but bf16 gates have few distinct values and large gates, whose products tend
+    to be a group's maximum, repeat); one bf16 step of the product is a relative 2^-8 .. 2^-7, which the smoothing division and the
+    division by 7 can each land on a coarser part of a binade.  Tolerance, stated here: at most 1e-2 of the
+    groups may have a different scale, none by more than 2^-6 relative (INT4, bf16 scales) or one step of
+    E4M3 (NVFP4); at most 1e-2 of the codes may differ, and every INT4 code must still be the
+    nearest one to the oracle's smoothed value under the kernel's own scale (half a step, plus one bf16 step
+    of the value); the projection to 1e-3 of its largest magnitude."""
+    M, K, R = 512, 1536, 32
+    announce(f"quantize fuse_glu random gates M={M} K={K} fp4={fp4}")
+    layer = synth.make_layer(128, K, R, seed=21, fp4=fp4)
+    g = torch.Generator().manual_seed(21)
+    x2 = _glu_pairs(synth.make_activations(M, K, seed=21).float(), 2.0 * torch.randn(M, K, generator=g))
+    codes, osc, la = _run(dev, x2, layer, fp4=fp4, fuse_glu=True)
+    want_codes, want_scales, want_la = olin.quantize_act_fuse_lora(x2, layer.proj_down, layer.smooth, fp4=fp4, fuse_glu=True)
+    assert codes.shape == want_codes.shape == (512, K)
+    if fp4:
+        sc_diff = (osc.view(torch.uint8).int() - want_scales.view(torch.uint8).int()).abs()
+        code_diff = codes.to(torch.uint8) != want_codes
+        assert sc_diff.max().item() <= 1
+    else:
+        sc_diff = (osc.float() - want_scales.float()).abs()
+        code_diff = codes != want_codes
+        assert (sc_diff <= 2.0**-6 * want_scales.float().abs()).all()
+        y = quant._smooth_divide(olin.glu_input(x2), layer.smooth, 0.0).float()
+        step = osc.float().t().repeat_interleave(64, dim=1)[:M]
+        assert ((codes[:M].float() * step - y).abs() <= 0.5 * step * (1 + 2.0**-6) + 2.0**-7 * y.abs()).all()
+    assert (sc_diff > 0).float().mean().item() <= 1e-2
+    assert code_diff.float().mean().item() <= 1e-2, f"{code_diff.sum().item()} codes differ"
+    assert (la - want_la).abs().max().item() <= 1e-3 * want_la.abs().max().item()
+    # and the padding rows stay zero
+    assert (codes[M:] == 0).all() and (la[M:] == 0).all()

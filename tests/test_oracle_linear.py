@@ -102,6 +102,31 @@ def _identity_layer(K, N, R, down_entry=None, up_entry=None, bias=None):
     return olin.FakeQuantLinear(wq, ws, torch.ones(K, dtype=torch.bfloat16), down, up, bias)
 
 
+def test_glu_input_literal_answers():
+    # pairs (value, gate).  silu(1) = 0.7310586 -> bf16 0.73046875 (187 * 2^-8); silu(-1) = -0.2689414 -> bf16
+    # -0.26953125 (138 * 2^-9); silu(2) = 1.7615942 -> bf16 1.7578125 (225 * 2^-7); silu(0) = 0
+    x = torch.tensor([[2.0, 1.0, 3.0, -1.0, 1.0, 2.0, 5.0, 0.0, 1.0078125, 1.0, -4.0, 1.0]], dtype=torch.bfloat16)
+    got = olin.glu_input(x)
+    # 2 * 0.73046875; 3 * -0.26953125 (exact in bf16); 1 * 1.7578125 (value and gate exchanged: not 1.4609375);
+    # 5 * 0; (1 + 2^-7) * 0.73046875 = 0.7361755 -> bf16 0.734375 (188 * 2^-8); -4 * 0.73046875
+    want = torch.tensor([[1.4609375, -0.80859375, 1.7578125, 0.0, 0.734375, -2.921875]])
+    assert got.dtype == torch.bfloat16 and torch.equal(got.float(), want)
+    # (the fifth pair also fixes that silu is rounded to bf16 before the product: with silu(1) kept in fp32 it would be
+    # (1 + 2^-7) * 0.7310586 = 0.73677 -> bf16 0.73828125)
+    # through the whole operator: the low-rank projection sees the product, not the raw columns
+    x = torch.zeros(1, 256, dtype=torch.bfloat16)
+    x[0, 0], x[0, 1] = 2.0, 1.0   # column 0 of the product: 1.4609375
+    x[0, 2], x[0, 3] = 3.0, -1.0  # column 1: -0.80859375
+    down = torch.zeros(128, 16, dtype=torch.bfloat16)
+    down[0, 0], down[1, 0], down[1, 1] = 1.0, 1.0, 2.0
+    codes, scales, la = olin.quantize_act_fuse_lora(x, down, None, fuse_glu=True)
+    assert codes.shape == (256, 128) and scales.shape == (2, 256)
+    assert la[0, 0].item() == 1.4609375 - 0.80859375 and la[0, 1].item() == -1.6171875
+    # group scale = bf16(1.4609375 / 7) = bf16(0.208705) = 0.208984375 (214 * 2^-10); codes rne(1.4609375 / 0.20870535) = 7,
+    # rne(-0.80859375 / 0.20870535 = -3.874) = -4
+    assert scales[0, 0].item() == 0.208984375 and codes[0, :3].tolist() == [7, -4, 0]
+
+
 def test_fake_quant_linear_literal():
     lin = _identity_layer(64, 64, 16, down_entry=(0, 0, 1.0), up_entry=(1, 0, 2.0), bias=torch.arange(64, dtype=torch.float32).to(torch.bfloat16))
     x = torch.zeros(2, 64)
