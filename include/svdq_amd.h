@@ -39,7 +39,7 @@ extern "C" {
 #define SVDQ_EUNSUPPORTED -2 /* valid request that this build does not implement */
 #define SVDQ_ELAUNCH -3      /* the HIP runtime refused the launch */
 
-#define SVDQ_ABI_VERSION 3
+#define SVDQ_ABI_VERSION 4
 
 int svdq_abi_version(void);
 const char *svdq_last_error(void);
@@ -182,6 +182,19 @@ typedef struct svdq_gemm_args {
     int32_t k_split;        /* 0: the library decides.  n > 0: split every output tile along K into n parts
                                whose partial sums meet in the workspace (1: never split); a tuning and
                                testing knob with no counterpart in the reference                      */
+    /* Separate q / k / v outputs of a fused QKV projection, in place of `out` (all NULL / 0 otherwise; needs
+     * rotary_emb).  Replaces EpiloguePackQKV, src/kernels/zgemm/epilogues.cuh:427-550, composed after the norm
+     * and rotation as in gemm_w4a4_launch_impl.cuh:380-397.  Each tensor is fp16 [heads = N/384][qkv_rows][128],
+     * head h at h * qkv_head_stride[i] elements (i = 0, 1, 2 for q, k, v: the tensors may be row ranges of larger
+     * ones, as in nunchaku/models/attention_processors/flux.py:139-160); values are fp16(bf16(x)) as in the
+     * reference (epilogues.cuh:446-453).  Rows [attn_tokens, qkv_rows) are written with the reference's mask
+     * values: 0 in q and v, NaN in k (epilogues.cuh:539-545).  Within a head the reference orders the values for
+     * its own attention kernel's matrix fragments; here they are plain [row][128], the order attention kernels
+     * on this hardware read.                                                                             */
+    void *out_q, *out_k, *out_v;
+    int64_t qkv_head_stride[3];
+    int64_t attn_tokens;    /* rows that hold tokens (the reference's actualM of this epilogue)              */
+    int64_t qkv_rows;       /* rows written per head, attn_tokens <= qkv_rows <= M_pad                       */
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);

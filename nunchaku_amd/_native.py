@@ -24,7 +24,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
-SVDQ_ABI_VERSION = 3
+SVDQ_ABI_VERSION = 4
 EXPORTED_SYMBOLS = [
     "svdq_abi_version", "svdq_last_error",
     "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
@@ -61,6 +61,8 @@ class GemmArgs(ctypes.Structure):
         ("fp4", ctypes.c_int32),
         ("norm_q", ctypes.c_void_p), ("norm_k", ctypes.c_void_p), ("rotary_emb", ctypes.c_void_p),
         ("rot_rows", ctypes.c_int64), ("norm_eps", ctypes.c_float), ("k_split", ctypes.c_int32),
+        ("out_q", ctypes.c_void_p), ("out_k", ctypes.c_void_p), ("out_v", ctypes.c_void_p),
+        ("qkv_head_stride", ctypes.c_int64 * 3), ("attn_tokens", ctypes.c_int64), ("qkv_rows", ctypes.c_int64),
     ]
 
 

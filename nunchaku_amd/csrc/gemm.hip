@@ -188,6 +188,9 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     p.rot_rows = (int)a->rot_rows;
     p.rope_cols = (int)(a->N / 3 * 2);
     p.norm_eps = a->norm_eps;
+    p.qkv.q = (uint16_t *)a->out_q; p.qkv.k = (uint16_t *)a->out_k; p.qkv.v = (uint16_t *)a->out_v;
+    p.qkv.stride_q = a->qkv_head_stride[0]; p.qkv.stride_k = a->qkv_head_stride[1]; p.qkv.stride_v = a->qkv_head_stride[2];
+    p.qkv.attn_tokens = (int)a->attn_tokens; p.qkv.rows = (int)a->qkv_rows;
     p.silu = a->fuse_silu != 0;
     p.gelu = a->qout != nullptr;  // the GELU is composed exactly when the next layer's input is produced (launch_impl.cuh:282-309)
 
@@ -253,6 +256,9 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     p.rot_rows = (int)a->rot_rows;
     p.rope_cols = (int)(a->N / 3 * 2);
     p.norm_eps = a->norm_eps;
+    p.qkv.q = (uint16_t *)a->out_q; p.qkv.k = (uint16_t *)a->out_k; p.qkv.v = (uint16_t *)a->out_v;
+    p.qkv.stride_q = a->qkv_head_stride[0]; p.qkv.stride_k = a->qkv_head_stride[1]; p.qkv.stride_v = a->qkv_head_stride[2];
+    p.qkv.attn_tokens = (int)a->attn_tokens; p.qkv.rows = (int)a->qkv_rows;
     p.silu = a->fuse_silu != 0;
     p.gelu = a->qout != nullptr;
 
@@ -302,7 +308,7 @@ int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
     SVDQ_REQUIRE(a->M_pad > 0 && a->M_pad % 256 == 0, "gemm: M_pad (%lld) must be a positive multiple of 256", (long long)a->M_pad);
     SVDQ_REQUIRE(a->N > 0 && a->N % 128 == 0, "gemm: N (%lld) must be a positive multiple of 128", (long long)a->N);
     SVDQ_REQUIRE(a->K > 0 && a->K % 128 == 0, "gemm: K (%lld) must be a positive multiple of 128", (long long)a->K);
-    SVDQ_REQUIRE(a->out || a->qout, "gemm: one of out / qout must be given");
+    SVDQ_REQUIRE(a->out || a->qout || a->out_q, "gemm: one of out / qout / out_q must be given");
     SVDQ_REQUIRE((a->lora_up != nullptr) == (a->lora_act_in != nullptr), "gemm: lora_up and lora_act_in go together");
     SVDQ_REQUIRE(a->R_up >= 0 && a->R_up % 16 == 0 && a->R_up <= 128, "gemm: R_up (%lld) must be a multiple of 16, at most 128", (long long)a->R_up);
     SVDQ_REQUIRE((a->R_up > 0) == (a->lora_up != nullptr), "gemm: R_up and lora_up disagree");
@@ -332,13 +338,29 @@ int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
     if (a->rotary_emb) {
         SVDQ_REQUIRE(a->norm_q && a->norm_k, "gemm: rotary_emb needs norm_q and norm_k");
         SVDQ_REQUIRE(a->N % 384 == 0, "gemm: rotary_emb needs N (%lld) to be three equal parts of 128-wide heads", (long long)a->N);
-        SVDQ_REQUIRE(a->out && !a->qout && a->N_out == a->N, "gemm: rotary_emb goes with a full-width `out` and no qout");
-        SVDQ_REQUIRE(a->rot_rows >= a->M_out && a->rot_rows <= a->M_pad && a->rot_rows % 32 == 0,
-                     "gemm: rotary_emb has %lld rows for %lld output rows (must cover them, in whole blocks of 32)", (long long)a->rot_rows, (long long)a->M_out);
+        SVDQ_REQUIRE(!a->qout, "gemm: rotary_emb goes without qout");
+        const long long covered = a->out_q ? a->attn_tokens : a->M_out;
+        if (a->out_q) {
+            // EpiloguePackQKV in place of the plain store (gemm_w4a4_launch_impl.cuh:380-397)
+            SVDQ_REQUIRE(!a->out && a->out_k && a->out_v, "gemm: out_q, out_k and out_v go together, without `out`");
+            SVDQ_REQUIRE(a->qkv_rows > 0 && a->qkv_rows <= a->M_pad && a->attn_tokens >= 0 && a->attn_tokens <= a->qkv_rows,
+                         "gemm: attn_tokens (%lld) <= qkv_rows (%lld) <= M_pad (%lld) does not hold", (long long)a->attn_tokens,
+                         (long long)a->qkv_rows, (long long)a->M_pad);
+            SVDQ_REQUIRE(a->qkv_head_stride[0] >= a->qkv_rows * 128 && a->qkv_head_stride[1] >= a->qkv_rows * 128 && a->qkv_head_stride[2] >= a->qkv_rows * 128,
+                         "gemm: a head of out_q / out_k / out_v holds qkv_rows x 128 values, the head strides are smaller");
+            SVDQ_REQUIRE(a->qkv_head_stride[0] % 8 == 0 && a->qkv_head_stride[1] % 8 == 0 && a->qkv_head_stride[2] % 8 == 0 &&
+                             ((uintptr_t)a->out_q | (uintptr_t)a->out_k | (uintptr_t)a->out_v) % 16 == 0,
+                         "gemm: out_q / out_k / out_v and their head strides must be 16-byte aligned");
+        } else {
+            SVDQ_REQUIRE(a->out && a->N_out == a->N, "gemm: rotary_emb goes with a full-width `out` (or with out_q, out_k, out_v)");
+        }
+        SVDQ_REQUIRE(a->rot_rows >= covered && a->rot_rows <= a->M_pad && a->rot_rows % 32 == 0,
+                     "gemm: rotary_emb has %lld rows for %lld output rows (must cover them, in whole blocks of 32)", (long long)a->rot_rows, covered);
         SVDQ_REQUIRE(((uintptr_t)a->rotary_emb % 16 == 0) && ((uintptr_t)a->norm_q % 8 == 0) && ((uintptr_t)a->norm_k % 8 == 0),
                      "gemm: rotary_emb / norm pointers are not aligned");
     } else {
         SVDQ_REQUIRE(!a->norm_q && !a->norm_k, "gemm: norm_q / norm_k need rotary_emb");
+        SVDQ_REQUIRE(!a->out_q && !a->out_k && !a->out_v, "gemm: out_q / out_k / out_v need rotary_emb (the reference composes them only there)");
     }
 
     int dev = 0;

@@ -504,6 +504,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         __builtin_amdgcn_wave_barrier();
         // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores.  Streaming stores: the
         // tile is not read again by this kernel.
+        if (NEXT && p.qkv.q && wcol0 < p.N) store_qkv_slab(p.qkv, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N / 3);
         if (p.out && interior) {  // no bounds to check: all slab reads first, then all stores
             u32x4_t d[8];
 #pragma unroll

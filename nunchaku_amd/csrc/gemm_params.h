@@ -25,6 +25,39 @@ constexpr int LDS_BYTES = NORMW_OFF + 4 * 512;
 constexpr int NORM_TARGET_EXP = 10;
 
 
+// Separate q / k / v outputs of a fused QKV projection (EpiloguePackQKV, epilogues.cuh:427-550): fp16
+// [heads][rows][128] each, head h at h * head_stride elements.  Rows [attn_tokens, rows) are written with
+// the mask value of the tensor: 0 for q and v, NaN for k.
+struct QkvOut {
+    uint16_t *q, *k, *v;      // null: the epilogue is not composed
+    long long stride_q, stride_k, stride_v;
+    int attn_tokens, rows;
+};
+
+// One wave writes a 32-row x 128-column bf16 slab (one head of q, k or v; rows `ld` elements apart in LDS)
+// to the tensor its columns belong to.  Values go bf16 -> fp32 -> fp16 as the reference's convert_half2
+// does (epilogues.cuh:446-453); 16 bytes per lane and pass, rows contiguous within a head.
+__device__ inline void store_qkv_slab(const QkvOut &o, const uint16_t *slab, int ld, int lane, int row0, int col0, int third) {
+    const int which = col0 / third, head = (col0 - which * third) >> 7;
+    uint16_t *base = which == 0 ? o.q : (which == 1 ? o.k : o.v);
+    const long long stride = which == 0 ? o.stride_q : (which == 1 ? o.stride_k : o.stride_v);
+    const uint32_t maskw = which == 1 ? 0x7FFF7FFFu : 0u;  // fp16 NaN pairs for k (epilogues.cuh:543), zeros for q and v
+    base += (size_t)head * stride;
+#pragma unroll
+    for (int pass = 0; pass < 8; pass++) {
+        const int rr = pass * 4 + (lane >> 4), cc = (lane & 15) * 8, m = row0 + rr;
+        const u32x4_t w = *(const u32x4_t *)(slab + rr * ld + cc);
+        u32x4_t d;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const _Float16 lo = (_Float16)bits_f32(w[j] << 16), hi = (_Float16)bits_f32(w[j] & 0xFFFF0000u);
+            d[j] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+            if (m >= o.attn_tokens) d[j] = maskw;
+        }
+        if (m < o.rows) __builtin_nontemporal_store(d, (u32x4_t *)(base + (size_t)m * 128 + cc));
+    }
+}
+
 struct GemmParams {
     const uint8_t *act;
     const uint16_t *ascales;
@@ -56,6 +89,7 @@ struct GemmParams {
     const float *rotary;              // fp32 [rot_rows/32][16][64 lanes][4], see svdq_gemm_args; null: no such epilogue
     int rot_rows, rope_cols;          // rope_cols = 2 N / 3: the columns of q and k
     float norm_eps;
+    QkvOut qkv;
 };
 
 
@@ -109,6 +143,7 @@ struct Params {
     const float *rotary;
     int rot_rows, rope_cols;
     float norm_eps;
+    QkvOut qkv;
 };
 }  // namespace g6
 

@@ -39,21 +39,27 @@ def fused_gelu_mlp(x: torch.Tensor, fc1, fc2, pad_size: int = 256) -> torch.Tens
 def fused_qkv_norm_rottary(x: torch.Tensor, proj, norm_q, norm_k, rotary_emb: torch.Tensor, output=None, attn_tokens: int = 0):
     """QKV projection with the RMS norm of q and k (per 128-wide head) and the rotary embedding fused
     into the GEMM epilogue (nunchaku/ops/fused.py:50-110).  ``norm_q`` / ``norm_k`` are modules with a
-    bf16 ``weight`` of 128 elements, ``rotary_emb`` is the table packed by ``pack_rotemb``.  The form
-    with a tuple ``output`` (q, k, v packed for the reference's attention kernel) is not built."""
-    if isinstance(output, tuple):
-        raise NotImplementedError("fused_qkv_norm_rottary: the (out_q, out_k, out_v) form is not built")
+    bf16 ``weight`` of 128 elements, ``rotary_emb`` is the table packed by ``pack_rotemb``.
+
+    ``output``: None or a bf16 tensor: q | k | v side by side, one row per token.  A tuple (q, k, v) of
+    fp16 [1, heads, tokens_pad, 128] tensors: the three apart, per head, rows from ``attn_tokens`` on
+    masked (see ``svdq_gemm_w4a4``)."""
     batch_size, seq_len, channels = x.shape
     x = x.view(batch_size * seq_len, channels)
     quantized_x, ascales, lora_act = proj.quantize(x)
+    t = proj.native_tensors()
+    common = dict(
+        act=quantized_x, wgt=t["qweight"], ascales=ascales, wscales=t["wscales"], lora_act_in=lora_act, lora_up=t["proj_up"],
+        bias=t["bias"], fp4=proj.precision == "nvfp4", alpha=proj.alpha, wcscales=t["wcscales"], norm_q=norm_q.weight,
+        norm_k=norm_k.weight, rotary_emb=rotary_emb, lora_scales=proj.lora_scales,
+    )
+    if isinstance(output, tuple):
+        if len(output) != 3:
+            raise ValueError("a tuple `output` is (q, k, v)")
+        svdq_gemm_w4a4(**common, out_q=output[0], out_k=output[1], out_v=output[2], attn_tokens=attn_tokens)
+        return output
     if output is None:
         output = torch.empty(quantized_x.shape[0], proj.out_features, dtype=x.dtype, device=x.device)
-    t = proj.native_tensors()
-    svdq_gemm_w4a4(
-        act=quantized_x, wgt=t["qweight"], out=output, ascales=ascales, wscales=t["wscales"],
-        lora_act_in=lora_act, lora_up=t["proj_up"], bias=t["bias"], fp4=proj.precision == "nvfp4",
-        alpha=proj.alpha, wcscales=t["wcscales"], norm_q=norm_q.weight, norm_k=norm_k.weight, rotary_emb=rotary_emb,
-        lora_scales=proj.lora_scales,
-    )
+    svdq_gemm_w4a4(**common, out=output)
     # (the reference views the padded buffer directly, which only works for token counts that need no padding)
     return output[: batch_size * seq_len].view(batch_size, seq_len, -1)

@@ -12,7 +12,7 @@ import torch
 from .. import _native as nv
 from .. import packing
 
-_NOT_BUILT = ("poolout", "out_vk", "out_linearattn", "out_q", "out_k", "out_v")
+_NOT_BUILT = ("poolout", "out_vk", "out_linearattn")
 NORM_EPS = 1e-6  # gemm_w4a4_launch_impl.cuh:374
 # Tuning / testing knob handed to the C ABI as ``k_split``: None lets the library decide, n > 0 splits
 # every output tile along K into n parts (1: never split).  No counterpart in the reference.
@@ -77,13 +77,16 @@ def svdq_gemm_w4a4(
     out      bf16 [M, N] (M <= M_pad);  qout / oscales / lora_act_out: inputs of the next layer, in
     which case a tanh-GELU is applied first (gemm_w4a4_launch_impl.cuh:282-309);
     norm_q / norm_k bf16 [128] and rotary_emb fp32 [B, M/B, 128] (packed by ``pack_rotemb``): RMS norm
-    and rotary embedding on the q and k thirds of ``out`` (launch_impl.cuh:347-402, the ``out`` form;
-    the ``out_q / out_k / out_v`` form that packs for the attention kernel is not built).
+    and rotary embedding on the q and k thirds of ``out`` (launch_impl.cuh:347-402);
+    out_q / out_k / out_v fp16 [1, heads, M_pad, 128] (row ranges of larger tensors are fine) with
+    attn_tokens: q, k, v apart, per head, in place of ``out``; rows from ``attn_tokens`` on hold 0 (q, v) and
+    NaN (k) as in the reference (epilogues.cuh:427-550).  Within a head the values are plain [row, 128]; the
+    reference orders them for its own attention kernel's matrix fragments.
     """
     local = locals()
     for name in _NOT_BUILT:
         if local[name] is not None:
-            raise NotImplementedError(f"svdq_gemm_w4a4: `{name}` (attention / linear-attention epilogues) is not built")
+            raise NotImplementedError(f"svdq_gemm_w4a4: `{name}` (linear-attention epilogue) is not built")
     for name in ("act", "wgt", "ascales", "wscales"):
         if local[name] is None:
             raise ValueError(f"svdq_gemm_w4a4: `{name}` is required")
@@ -92,8 +95,11 @@ def svdq_gemm_w4a4(
         raise ValueError("lora_up and lora_act_in must be given together")
     if (lora_down is None) != (lora_act_out is None):
         raise ValueError("lora_down and lora_act_out must be given together")
-    if out is None and qout is None:
-        raise ValueError("one of out / qout is required")
+    qkv = (out_q, out_k, out_v)
+    if any(t is not None for t in qkv) and (any(t is None for t in qkv) or rotary_emb is None or out is not None):
+        raise ValueError("out_q, out_k and out_v go together, with rotary_emb and without `out` (launch_impl.cuh:380-397)")
+    if out is None and qout is None and out_q is None:
+        raise ValueError("one of out / qout / (out_q, out_k, out_v) is required")
     if qout is not None and (oscales is None or smooth_factor is None):
         raise ValueError("qout needs oscales and smooth_factor")
     if rotary_emb is not None and (norm_q is None or norm_k is None):
@@ -163,8 +169,22 @@ def svdq_gemm_w4a4(
             nv.require_gpu(t, name)
             if t.dtype != torch.bfloat16 or t.numel() != 128 or not t.is_contiguous():
                 raise ValueError(f"{name} must be a contiguous bf16 vector of 128 elements (one head)")
-        if out is None or out.shape[-1] != N:
+        if out_q is None and (out is None or out.shape[-1] != N):
             raise ValueError("rotary_emb needs a full-width `out`")
+    qkv_strides = (0, 0, 0)
+    if out_q is not None:
+        if N % 384:
+            raise ValueError("out_q / out_k / out_v need N to be three equal parts of 128-wide heads")
+        for name, t in zip(("out_q", "out_k", "out_v"), qkv):
+            if not t.is_cuda:
+                raise RuntimeError(f"{name} must live on a GPU (got {t.device}); this path has no CPU implementation")
+            if t.dtype != torch.float16 or t.device != dev or tuple(t.shape) != (1, N // 384, M_pad, 128) or t.stride(3) != 1 or t.stride(2) != 128:
+                raise ValueError(
+                    f"{name} must be float16 [1, {N // 384}, {M_pad}, 128] with contiguous rows (one batch: the reference places row "
+                    f"block b of the GEMM at row block b of every head, epilogues.cuh:535), got {tuple(t.shape)} {t.dtype}")
+        if not 0 <= attn_tokens <= M_pad:
+            raise ValueError(f"attn_tokens must lie in [0, {M_pad}]")
+        qkv_strides = tuple(t.stride(1) for t in qkv)
 
     n_sc = max(1, math.ceil(rank_up / 16))
     sc = (ctypes.c_float * n_sc)(*[float(lora_scales[i]) if i < len(lora_scales) else 0.0 for i in range(n_sc)])
@@ -181,6 +201,8 @@ def svdq_gemm_w4a4(
         alpha=float(alpha), act_unsigned=int(act_unsigned), fuse_silu=int(fuse_silu), fp4=int(fp4),
         norm_q=nv.ptr(norm_q), norm_k=nv.ptr(norm_k), rotary_emb=nv.ptr(rot_n),
         rot_rows=0 if rot_n is None else rot_n.shape[0], norm_eps=NORM_EPS, k_split=int(K_SPLIT or 0),
+        out_q=nv.ptr(out_q), out_k=nv.ptr(out_k), out_v=nv.ptr(out_v), qkv_head_stride=(ctypes.c_int64 * 3)(*qkv_strides),
+        attn_tokens=int(attn_tokens) if out_q is not None else 0, qkv_rows=M_pad if out_q is not None else 0,
     )
     with torch.cuda.device(dev):  # the library launches on the current device
         entry = nv.lib().svdq_gemm_w4a4_noalloc if NO_ALLOC else nv.lib().svdq_gemm_w4a4

@@ -169,3 +169,27 @@ def rmsnorm_rope(out: torch.Tensor, norm_q: torch.Tensor, norm_k: torch.Tensor, 
         r = torch.stack((a * cos[:, None, :] - b * sin[:, None, :], a * sin[:, None, :] + b * cos[:, None, :]), dim=-1)
         x[:, part * third:(part + 1) * third] = r.reshape(M, third)
     return x.to(torch.float32)
+
+
+def pack_qkv(out: torch.Tensor, attn_tokens: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """EpiloguePackQKV (src/kernels/zgemm/epilogues.cuh:427-550), composed after the norm and rotation
+    (gemm_w4a4_launch_impl.cuh:380-397), as logical tensors.
+
+    out fp32 [M_pad, N], N = 3 * heads * 128, the epilogue's input before its bf16 rounding.  Column block b of
+    128 is head ``b % heads`` of q (b < heads), k (b < 2 heads) or v (:517-533).  Values are rounded to bf16
+    (the GEMM's tile type) and converted to fp16 through fp32 (``convert_half2``, :446-453).  Rows from
+    ``attn_tokens`` on are replaced by the mask value of the tensor: 0 for q and v, NaN for k (:482-492,
+    :539-545).  Returns three fp16 [1, heads, M_pad, 128] tensors holding [row, dim] per head; the reference
+    stores the same values in the order of its attention kernel's matrix fragments (:494-512), which is
+    private to that kernel and not restated.
+    """
+    M_pad, N = out.shape
+    assert N % 384 == 0
+    heads = N // 384
+    x = out.to(torch.bfloat16).to(torch.float32).to(torch.float16)
+    parts = []
+    for i, mask in enumerate((0.0, float("nan"), 0.0)):
+        t = x[:, i * heads * 128:(i + 1) * heads * 128].reshape(M_pad, heads, 128).permute(1, 0, 2).contiguous()
+        t[:, attn_tokens:, :] = mask
+        parts.append(t[None])
+    return tuple(parts)

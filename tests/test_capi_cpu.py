@@ -29,11 +29,41 @@ def test_header_symbols_are_exported(lib):
     assert int(re.search(r"#define SVDQ_ABI_VERSION (\d+)", header).group(1)) == nv.SVDQ_ABI_VERSION
 
 
-def test_struct_sizes_match_header_layout():
-    # 6 pointers + 4 int64 + 2 int32 ; 16 pointers + 7 int64 + float + 3 int32, then 3 pointers + int64 +
-    # float + int32
-    assert ctypes.sizeof(nv.QuantizeArgs) == 6 * 8 + 4 * 8 + 2 * 4
-    assert ctypes.sizeof(nv.GemmArgs) == 16 * 8 + 7 * 8 + 4 * 4 + 3 * 8 + 8 + 8
+def test_struct_sizes_match_header_layout(tmp_path):
+    """The ctypes mirrors against the header itself: a C program that includes it prints the size of every
+    argument block and the offset of every field, compiled with the host compiler."""
+    import re
+    import shutil
+    import subprocess
+    from pathlib import Path
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no host C compiler")
+    header = Path(__file__).resolve().parent.parent / "include" / "svdq_amd.h"
+    mirrors = {"svdq_quantize_args": nv.QuantizeArgs, "svdq_gemm_args": nv.GemmArgs, "svdq_awq_gemv_args": nv.AwqGemvArgs}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{header}"', 'int main(void) {']
+    for cname, mirror in mirrors.items():
+        lines.append(f'printf("{cname} %zu\\n", sizeof({cname}));')
+        for fname, *_ in mirror._fields_:
+            lines.append(f'printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines.append("return 0; }")
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run([cc, str(src), "-o", str(exe)], check=True, capture_output=True)
+    out = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, mirror in mirrors.items():
+        assert int(out[cname]) == ctypes.sizeof(mirror), cname
+        for fname, *_ in mirror._fields_:
+            assert int(out[f"{cname}.{fname}"]) == getattr(mirror, fname).offset, f"{cname}.{fname}"
+    # and no field of the header is missing from the mirror
+    text = header.read_text()
+    for cname, mirror in mirrors.items():
+        body = text[text.index(f"typedef struct {cname}"):text.index(f"}} {cname};")]
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        names = re.findall(r"[\s\*]([A-Za-z_][A-Za-z0-9_]*)\s*(?:\[\d+\])?\s*[,;]", body)
+        assert set(names) == {f[0] for f in mirror._fields_}, cname
 
 
 def test_quantize_rejects_bad_arguments(lib):
@@ -143,7 +173,7 @@ def test_python_wrappers_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU"):
         svdq_quantize_w4a4_act_fuse_lora(x, lora_down=torch.zeros(128, 16, dtype=torch.bfloat16))
     with pytest.raises(NotImplementedError):
-        svdq_gemm_w4a4(act=x, wgt=x, out_q=x)
+        svdq_gemm_w4a4(act=x, wgt=x, out_vk=x)
     with pytest.raises(RuntimeError, match="GPU"):
         svdq_gemm_w4a4(act=x.view(torch.uint8), wgt=x.view(torch.int8), ascales=x, wscales=x, out=x)
 

@@ -57,3 +57,30 @@ def test_rotation_keeps_the_norm_and_quarter_turn_swaps():
     base = olin.rmsnorm_rope(x, ones, ones, torch.stack((torch.zeros(M, 64), torch.ones(M, 64)), -1).reshape(M, 128))
     assert torch.allclose(q[:, 0:256:2], -base[:, 1:256:2], atol=1e-6)
     assert torch.allclose(q[:, 1:256:2], base[:, 0:256:2], atol=1e-6)
+
+
+def test_pack_qkv_literal_answers():
+    """Two heads, four rows, three tokens.  Which column goes to which tensor and head, the two roundings and
+    the mask values are written out by hand."""
+    from oracle import linear as olin
+
+    out = torch.zeros(4, 768)
+    out[0, 0] = 1.0            # q, head 0, dim 0
+    out[0, 128 + 5] = 2.0      # q, head 1, dim 5
+    out[1, 256 + 7] = 3.0      # k, head 0, dim 7
+    out[2, 384 + 127] = -4.0   # k, head 1, dim 127
+    out[2, 512] = 5.0          # v, head 0, dim 0
+    out[0, 640 + 64] = 1.00390625   # v, head 1: 1 + 2^-8 is a bf16 tie, rounds to 1.0 although fp16 could hold it
+    out[1, 640] = 70000.0      # bf16 70144, beyond fp16: +inf
+    out[1, 1] = 2.0**-25       # the midpoint of the fp16 subnormals 0 and 2^-24: ties to even, 0 ...
+    out[1, 2] = 1.5 * 2.0**-24  # ... and the midpoint of 2^-24 and 2 * 2^-24 goes to 2 * 2^-24
+    out[3] = 9.0               # row 3 is padding
+    q, k, v = olin.pack_qkv(out, attn_tokens=3)
+    assert q.shape == k.shape == v.shape == (1, 2, 4, 128) and q.dtype == torch.float16
+    assert q[0, 0, 0, 0] == 1.0 and q[0, 1, 0, 5] == 2.0 and q[0, 0, 0].abs().sum() == 1.0
+    assert k[0, 0, 1, 7] == 3.0 and k[0, 1, 2, 127] == -4.0
+    assert v[0, 0, 2, 0] == 5.0 and v[0, 1, 0, 64] == 1.0
+    assert torch.isinf(v[0, 1, 1, 0]) and v[0, 1, 1, 0] > 0
+    assert q[0, 0, 1, 1] == 0.0 and q[0, 0, 1, 2].item() == 2.0**-23
+    assert (q[0, :, 3] == 0).all() and (v[0, :, 3] == 0).all() and torch.isnan(k[0, :, 3]).all()
+    assert not torch.isnan(k[0, :, :3]).any()
