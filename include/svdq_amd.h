@@ -195,6 +195,17 @@ typedef struct svdq_gemm_args {
     int64_t qkv_head_stride[3];
     int64_t attn_tokens;    /* rows that hold tokens (the reference's actualM of this epilogue)              */
     int64_t qkv_rows;       /* rows written per head, attn_tokens <= qkv_rows <= M_pad                       */
+    /* Linear attention (INT4 only; NULL / 0 otherwise).  Replaces EpilogueLiteLA,
+     * src/kernels/zgemm/epilogues.cuh:552-681, selected as in gemm_w4a4_launch_impl.cuh:311-345 (with `out` alone,
+     * after bias and low-rank up).  N = 3 * heads * 32.  Columns [0, N/3) are q: `out` = bf16 [M_pad, N/3] receives
+     * relu(q) (the reference's out_linearattn).  The other columns hold, per head, 32 of k then 32 of v, and
+     *   out_vk[b][head][i][j] = sum over the vk_rows rows of batch entry b of v[row][i] * relu(k[row][j]),  i < 32,
+     *   out_vk[b][head][32][j] = sum of relu(k[row][j]),
+     * on the bf16-rounded values, accumulated in fp32.  Every row of the GEMM counts, padding rows included, as in
+     * the reference.  The library clears out_vk on `stream` first (the reference's launcher does, :335); sums of
+     * different row blocks arrive through fp32 atomics in no fixed order, as the reference's do (:649).       */
+    float *out_vk;          /* fp32 [M_pad / vk_rows][2 N / 3 / 64][33][32]                                   */
+    int64_t vk_rows;        /* rows per batch entry: a multiple of 256 that divides M_pad                     */
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
@@ -211,6 +222,16 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
  * in time on one GPU race with each other.  What a launch needs to be zero at its start is cleared by a
  * fill kernel on `stream` first. */
 int svdq_gemm_w4a4_noalloc(const svdq_gemm_args *args, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Linear attention, second half: q[b][t][h][:] <- (vk[b][h][:32] q) / (vk[b][h][32] . q + eps), in place.
+ * Replaces kernels::linearattn_vk_mul_q (src/kernels/zgemm/zgemm.h:37 ->
+ * gemm_w4a4_launch_impl.cuh:427-448, kernel epilogues.cuh:683-744; the reference passes eps = 1e-6).
+ * q: bf16 [batch][tokens_pad][heads][32], the `out` of svdq_gemm_w4a4 with out_vk; vk: its out_vk.
+ * Rows num_tokens .. tokens_pad of every batch entry are left as they are.
+ * ------------------------------------------------------------------------------------------ */
+int svdq_linearattn_vk_mul_q(void *q, const float *vk, int64_t batch, int64_t num_tokens, int64_t tokens_pad, int64_t heads,
+                             float eps, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * AWQ W4A16 GEMV (the other quantized linear of the reference's models: modulation layers, text

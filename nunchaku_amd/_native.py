@@ -18,7 +18,7 @@ import torch
 _PKG_DIR = Path(__file__).resolve().parent
 _CSRC = _PKG_DIR / "csrc"
 LIB_PATH = _PKG_DIR / "libsvdq_amd.so"
-SOURCES = ["repack.hip", "quantize.hip", "gemm.hip", "awq_gemv.hip"]
+SOURCES = ["repack.hip", "quantize.hip", "gemm.hip", "awq_gemv.hip", "litela.hip"]
 HIPCC_FLAGS = [
     "-shared", "-fPIC", "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = [
     "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
     "svdq_repack_smooth", "svdq_repack_lora_down", "svdq_repack_lora_up", "svdq_repack_rotemb",
     "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4", "svdq_gemm_w4a4_noalloc", "svdq_awq_gemv_w4a16",
+    "svdq_linearattn_vk_mul_q",
 ]
 
 
@@ -63,6 +64,7 @@ class GemmArgs(ctypes.Structure):
         ("rot_rows", ctypes.c_int64), ("norm_eps", ctypes.c_float), ("k_split", ctypes.c_int32),
         ("out_q", ctypes.c_void_p), ("out_k", ctypes.c_void_p), ("out_v", ctypes.c_void_p),
         ("qkv_head_stride", ctypes.c_int64 * 3), ("attn_tokens", ctypes.c_int64), ("qkv_rows", ctypes.c_int64),
+        ("out_vk", ctypes.c_void_p), ("vk_rows", ctypes.c_int64),
     ]
 
 
@@ -140,6 +142,7 @@ def lib() -> ctypes.CDLL:
         L.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.svdq_gemm_w4a4_noalloc.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), vp]
+        L.svdq_linearattn_vk_mul_q.argtypes = [vp, vp, i64, i64, i64, i64, ctypes.c_float, vp]
         for name in EXPORTED_SYMBOLS:
             getattr(L, name)
             if name not in ("svdq_last_error",):

@@ -191,6 +191,8 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     p.qkv.q = (uint16_t *)a->out_q; p.qkv.k = (uint16_t *)a->out_k; p.qkv.v = (uint16_t *)a->out_v;
     p.qkv.stride_q = a->qkv_head_stride[0]; p.qkv.stride_k = a->qkv_head_stride[1]; p.qkv.stride_v = a->qkv_head_stride[2];
     p.qkv.attn_tokens = (int)a->attn_tokens; p.qkv.rows = (int)a->qkv_rows;
+    p.vk = a->out_vk;
+    p.vk_rows = (int)a->vk_rows;
     p.silu = a->fuse_silu != 0;
     p.gelu = a->qout != nullptr;  // the GELU is composed exactly when the next layer's input is produced (launch_impl.cuh:282-309)
 
@@ -208,7 +210,12 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
         if (kparts < 1) kparts = 1;
     }
     p.kparts = kparts;
-    const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu;
+    const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu || a->out_vk != nullptr;
+    if (p.vk) {
+        // the sums start at zero (the reference's launcher clears the tensor too, gemm_w4a4_launch_impl.cuh:335)
+        const size_t n = (size_t)(p.M_pad / p.vk_rows) * (p.N / 3 * 2 / 64) * g6::VK_HEAD_FLOATS;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, p.vk, (int64_t)n);
+    }
     const size_t cnt_bytes = (size_t)ntiles * 4, lcnt_bytes = (size_t)mblocks * 4;
     const size_t fix_bytes = p.next_down ? (size_t)p.M_pad * p.R_down * 8 : 0;
     const size_t part_bytes = kparts > 1 ? (size_t)ntiles * kparts * g6::BM * g6::BN * 4 : 0;
@@ -316,8 +323,21 @@ int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
     if (a->out) {
         SVDQ_REQUIRE(a->M_out > 0 && a->M_out <= a->M_pad && a->M_pad - a->M_out < 256, "gemm: M_out (%lld) does not fit M_pad (%lld)",
                      (long long)a->M_out, (long long)a->M_pad);
-        SVDQ_REQUIRE(a->N_out > 0 && a->N_out <= a->N && a->N - a->N_out < 128 && a->N_out % 8 == 0,
-                     "gemm: N_out (%lld) must be a multiple of 8 within 128 of N (%lld)", (long long)a->N_out, (long long)a->N);
+        if (a->out_vk) {
+            SVDQ_REQUIRE(a->N_out * 3 == a->N && a->M_out == a->M_pad, "gemm: with out_vk, `out` is the q third of all rows: [M_pad, N/3]");
+        } else {
+            SVDQ_REQUIRE(a->N_out > 0 && a->N_out <= a->N && a->N - a->N_out < 128 && a->N_out % 8 == 0,
+                         "gemm: N_out (%lld) must be a multiple of 8 within 128 of N (%lld)", (long long)a->N_out, (long long)a->N);
+        }
+    }
+    if (a->out_vk) {
+        // EpilogueLiteLA (gemm_w4a4_launch_impl.cuh:311-345)
+        if (a->fp4) return fail(SVDQ_EUNSUPPORTED, "gemm: out_vk (linear attention) is built for INT4 operands only");
+        SVDQ_REQUIRE(a->out && !a->qout && !a->rotary_emb && !a->next_lora_down && !a->fuse_silu, "gemm: out_vk goes with `out` (the q third) alone");
+        SVDQ_REQUIRE(a->N % 384 == 0, "gemm: out_vk needs N (%lld) to be three equal parts of whole 128-column blocks", (long long)a->N);
+        SVDQ_REQUIRE(a->vk_rows > 0 && a->vk_rows % 256 == 0 && a->M_pad % a->vk_rows == 0,
+                     "gemm: vk_rows (%lld) must be a multiple of 256 that divides M_pad (%lld)", (long long)a->vk_rows, (long long)a->M_pad);
+        SVDQ_REQUIRE((uintptr_t)a->out_vk % 16 == 0, "gemm: out_vk must be 16-byte aligned");
     }
     SVDQ_REQUIRE(((uintptr_t)a->act | (uintptr_t)a->wgt | (uintptr_t)a->ascales | (uintptr_t)a->wscales | (uintptr_t)a->out |
                   (uintptr_t)a->lora_act_in | (uintptr_t)a->lora_up) % 16 == 0, "gemm: pointers must be 16-byte aligned");

@@ -339,6 +339,10 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
         coltab[tid] = cf;
         coltab[256 + tid] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+        if (NEXT && p.vk) {
+            float *vkz = (float *)(lds + EP_VK);
+            for (int i = tid; i < 2 * 2 * VK_HEAD_FLOATS; i += 256) vkz[i] = 0.f;
+        }
         if (NEXT && p.rotary && tid < 128) {
             // RMS-norm weights of the heads the two column halves are (q below N/3, k below 2N/3)
             ((float *)(lds + EP_NORMW))[tid] = bf16_bits_to_f32((n0 < p.rope_cols / 2 ? p.norm_q : p.norm_k)[tid]);
@@ -487,6 +491,13 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
 #pragma unroll
                 for (int e = 0; e < 16; e++) v[nt][e] = gelu_tanh(v[nt][e]);
         }
+        if (NEXT && p.vk && wcol0 < p.N / 3) {
+            // the q third of a linear-attention projection is stored after a ReLU (epilogues.cuh:662-674)
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) v[nt][e] = __builtin_fmaxf(v[nt][e], 0.f);
+        }
         // bf16 tile -> per-wave LDS slab (32 rows x 128 columns), four columns per write: every later
         // consumer reads whole rows
 #pragma unroll
@@ -504,6 +515,47 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         __builtin_amdgcn_wave_barrier();
         // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores.  Streaming stores: the
         // tile is not read again by this kernel.
+        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) {
+            // EpilogueLiteLA::apply_litela (epilogues.cuh:572-655) on this slab: the wave's 128 columns are two
+            // heads of [k 32 | v 32].  vk[i][j] = sum over the 32 rows of v[row][i] * relu(k[row][j]) on the
+            // matrix cores (the rows are the contraction index: both operands are read down the columns of
+            // the slab), row 32 = sum of relu(k[row][j]).  The slabs and waves of the workgroup that share a
+            // head add up in LDS.
+            float *vkacc = (float *)(lds + EP_VK) + wn * (2 * VK_HEAD_FLOATS);
+            const int j = lane & 31, kb = lane >> 5;
+#pragma unroll
+            for (int hd = 0; hd < 2; hd++) {
+                float16_t d;
+#pragma unroll
+                for (int e = 0; e < 16; e++) d[e] = 0.f;
+                float ks = 0.f;
+#pragma unroll
+                for (int st = 0; st < 2; st++) {
+                    u32x4_t kw, vw;
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2) {
+                        uint32_t kk[2], vv[2];
+#pragma unroll
+                        for (int f = 0; f < 2; f++) {
+                            const uint16_t *rowp = slab + (16 * st + 8 * kb + e + f) * OUT_LD + hd * 64 + j;
+                            kk[f] = rowp[0];
+                            vv[f] = rowp[32];
+                            if (kk[f] & 0x8000u) kk[f] = 0;  // ReLU on the bf16 value
+                            ks += bits_f32(kk[f] << 16);
+                        }
+                        kw[e / 2] = kk[0] | (kk[1] << 16);
+                        vw[e / 2] = vv[0] | (vv[1] << 16);
+                    }
+                    d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vw), __builtin_bit_cast(bf16x8_t, kw), d, 0, 0, 0);
+                }
+                ks += __shfl_xor(ks, 32);
+                float *dst = vkacc + hd * VK_HEAD_FLOATS;
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    __hip_atomic_fetch_add(dst + ((e >> 2) * 8 + kb * 4 + (e & 3)) * 32 + j, d[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (kb == 0) __hip_atomic_fetch_add(dst + 32 * 32 + j, ks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
         if (NEXT && p.qkv.q && wcol0 < p.N) store_qkv_slab(p.qkv, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N / 3);
         if (p.out && interior) {  // no bounds to check: all slab reads first, then all stores
             u32x4_t d[8];
@@ -607,6 +659,21 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     __builtin_amdgcn_sched_barrier(0);
     slab_epilogue(std::integral_constant<int, 0>{});
     slab_epilogue(std::integral_constant<int, 1>{});
+
+    if (NEXT && p.vk) {
+        // the tile's sums join those of the other row blocks (the reference's reduce_add, epilogues.cuh:649: the
+        // order of arrival decides the rounding there as here)
+        __syncthreads();
+        const float *vkall = (const float *)(lds + EP_VK);
+        const int third = p.N / 3, heads = 2 * third / 64, batch = m0 / p.vk_rows;
+        for (int i = tid; i < 2 * 2 * VK_HEAD_FLOATS; i += 256) {
+            const int half = i / (2 * VK_HEAD_FLOATS), rem = i - half * (2 * VK_HEAD_FLOATS);
+            const int col0 = n0 + half * 128;
+            if (col0 < third || col0 >= p.N) continue;
+            const int head = (col0 - third) / 64 + rem / VK_HEAD_FLOATS;
+            unsafeAtomicAdd(p.vk + ((size_t)batch * heads + head) * VK_HEAD_FLOATS + rem % VK_HEAD_FLOATS, vkall[i]);
+        }
+    }
 
     if (NEXT && p.next_down) {
         // The workgroup that adds the last column block's share to a block of 128 rows turns the

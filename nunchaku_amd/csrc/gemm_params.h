@@ -110,8 +110,10 @@ constexpr int EP_TAB = 4 * SLAB_BYTES;     // float cf[256], bias[256]
 constexpr int EP_NORMW = EP_TAB + 2048;    // 4 waves x float [128]: RMS-norm weights of the wave's head
 constexpr int EP_FLAG = EP_NORMW + 2048;   // one word handed from thread 0 to the workgroup
 constexpr int EP_RED = EP_FLAG + 16;       // [2 row halves][2][64 lanes] x float4: the two column halves' low-rank sums meet here
+constexpr int EP_VK = EP_RED + 2 * 2 * 64 * 16;  // [2 column halves][2 heads][33][32] floats: linear-attention sums of the tile
+constexpr int VK_HEAD_FLOATS = 33 * 32;
 constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-static_assert(EP_RED + 2 * 2 * 64 * 16 <= LDS_BYTES, "the epilogue must fit the ring");
+static_assert(EP_VK + 2 * 2 * VK_HEAD_FLOATS * 4 <= LDS_BYTES, "the epilogue must fit the ring");
 
 struct Params {
     const uint8_t *act;        // fragments [M_pad/128][K/64][4]
@@ -144,6 +146,11 @@ struct Params {
     int rot_rows, rope_cols;
     float norm_eps;
     QkvOut qkv;
+    // linear attention (EpilogueLiteLA, epilogues.cuh:552-681; next-layer variant only): columns [0, N/3) are q,
+    // stored through `out` after a ReLU; the rest is [head][k 32 | v 32]; vk[batch][head][i][j] += sum over the
+    // tile's rows of v[i] relu(k[j]) (i < 32) and of relu(k[j]) (i = 32)
+    float *vk;           // fp32 [batch][2 N / 3 / 64][33][32], zero before the launch; null: no such epilogue
+    int vk_rows;         // rows per batch entry, a multiple of 256
 };
 }  // namespace g6
 

@@ -63,3 +63,27 @@ def fused_qkv_norm_rottary(x: torch.Tensor, proj, norm_q, norm_k, rotary_emb: to
     svdq_gemm_w4a4(**common, out=output)
     # (the reference views the padded buffer directly, which only works for token counts that need no padding)
     return output[: batch_size * seq_len].view(batch_size, seq_len, -1)
+
+
+def linearattn_vk_mul_q(q: torch.Tensor, vk: torch.Tensor, num_tokens: int | None = None, eps: float = 1e-6) -> torch.Tensor:
+    """Second half of the linear attention: ``q[b, t, h] <- (vk[b, h, :32] @ q[b, t, h]) / (vk[b, h, 32] . q[b, t, h] + eps)``
+    in place (kernels::linearattn_vk_mul_q, gemm_w4a4_launch_impl.cuh:427-448).  q bf16 [B, tokens_pad, heads * 32]
+    (``out_linearattn`` of ``svdq_gemm_w4a4``), vk fp32 [B, heads, 33, 32] (its ``out_vk``); only the first
+    ``num_tokens`` rows of every batch entry are touched (all by default, as in the reference)."""
+    import ctypes
+
+    from .. import _native as nv
+
+    nv.require_gpu(q, "q")
+    nv.require_gpu(vk, "vk")
+    if q.dim() != 3 or vk.dim() != 4 or q.dtype != torch.bfloat16 or vk.dtype != torch.float32:
+        raise ValueError("q is bf16 [B, tokens_pad, heads * 32] and vk fp32 [B, heads, 33, 32]")
+    B, tokens_pad, width = q.shape
+    heads = vk.shape[1]
+    if tuple(vk.shape) != (B, heads, 33, 32) or width != heads * 32 or vk.device != q.device:
+        raise ValueError(f"vk has shape {tuple(vk.shape)}; q [{B}, {tokens_pad}, {width}] takes [{B}, {width // 32}, 33, 32] on the same device")
+    num_tokens = tokens_pad if num_tokens is None else int(num_tokens)
+    with torch.cuda.device(q.device):
+        nv.check(nv.lib().svdq_linearattn_vk_mul_q(q.data_ptr(), vk.data_ptr(), B, num_tokens, tokens_pad, heads, ctypes.c_float(eps),
+                                                   nv.stream_ptr(q.device)))
+    return q

@@ -12,7 +12,7 @@ import torch
 from .. import _native as nv
 from .. import packing
 
-_NOT_BUILT = ("poolout", "out_vk", "out_linearattn")
+_NOT_BUILT = ("poolout",)
 NORM_EPS = 1e-6  # gemm_w4a4_launch_impl.cuh:374
 # Tuning / testing knob handed to the C ABI as ``k_split``: None lets the library decide, n > 0 splits
 # every output tile along K into n parts (1: never split).  No counterpart in the reference.
@@ -82,11 +82,17 @@ def svdq_gemm_w4a4(
     attn_tokens: q, k, v apart, per head, in place of ``out``; rows from ``attn_tokens`` on hold 0 (q, v) and
     NaN (k) as in the reference (epilogues.cuh:427-550).  Within a head the values are plain [row, 128]; the
     reference orders them for its own attention kernel's matrix fragments.
+    out_linearattn bf16 [B, tokens_pad, N/3] with out_vk fp32 [B, heads, 33, 32] (N = 3 * heads * 32, tokens_pad a
+    multiple of 256, INT4 only): linear attention (launch_impl.cuh:311-345): relu(q) goes to out_linearattn;
+    out_vk[b, h, i, j] = sum over tokens of v[i] * relu(k[j]) (i < 32) and of relu(k[j]) (i = 32), where the
+    columns after q hold, per head, 32 of k then 32 of v.  out_vk is cleared first.
     """
     local = locals()
     for name in _NOT_BUILT:
         if local[name] is not None:
-            raise NotImplementedError(f"svdq_gemm_w4a4: `{name}` (linear-attention epilogue) is not built")
+            # the reference's signature carries it, but no branch of its launcher consumes it any more (the epilogue
+            # that did is commented out, gemm_w4a4_launch_impl.cuh:362-373)
+            raise NotImplementedError(f"svdq_gemm_w4a4: `{name}` is not built (the reference ignores it)")
     for name in ("act", "wgt", "ascales", "wscales"):
         if local[name] is None:
             raise ValueError(f"svdq_gemm_w4a4: `{name}` is required")
@@ -98,8 +104,15 @@ def svdq_gemm_w4a4(
     qkv = (out_q, out_k, out_v)
     if any(t is not None for t in qkv) and (any(t is None for t in qkv) or rotary_emb is None or out is not None):
         raise ValueError("out_q, out_k and out_v go together, with rotary_emb and without `out` (launch_impl.cuh:380-397)")
-    if out is None and qout is None and out_q is None:
-        raise ValueError("one of out / qout / (out_q, out_k, out_v) is required")
+    if (out_vk is None) != (out_linearattn is None):
+        raise ValueError("out_vk and out_linearattn go together")  # the reference asserts it (launch_impl.cuh:313)
+    if out_vk is not None:
+        if out is not None or qout is not None or out_q is not None or rotary_emb is not None or fuse_silu:
+            raise ValueError("out_vk / out_linearattn go without out, qout, out_q and rotary_emb (launch_impl.cuh:282-417 picks one branch)")
+        if fp4:
+            raise NotImplementedError("the linear-attention epilogue is built for INT4 layers only")
+    if out is None and qout is None and out_q is None and out_vk is None:
+        raise ValueError("one of out / qout / (out_q, out_k, out_v) / (out_vk, out_linearattn) is required")
     if qout is not None and (oscales is None or smooth_factor is None):
         raise ValueError("qout needs oscales and smooth_factor")
     if rotary_emb is not None and (norm_q is None or norm_k is None):
@@ -186,6 +199,20 @@ def svdq_gemm_w4a4(
             raise ValueError(f"attn_tokens must lie in [0, {M_pad}]")
         qkv_strides = tuple(t.stride(1) for t in qkv)
 
+    vk_rows = 0
+    if out_vk is not None:
+        if N % 384:
+            raise ValueError("out_vk needs N to be three equal parts of whole 128-column blocks")
+        heads = N // 96
+        if out_linearattn.dim() != 3 or out_vk.dim() != 4:
+            raise ValueError("out_linearattn is [B, tokens_pad, N/3] and out_vk [B, heads, 33, 32]")
+        B, vk_rows = out_linearattn.shape[0], out_linearattn.shape[1]
+        _expect("out_linearattn", out_linearattn, (B, vk_rows, N // 3), torch.bfloat16, dev)
+        _expect("out_vk", out_vk, (B, heads, 33, 32), torch.float32, dev)
+        if vk_rows % 256 or B * vk_rows != M_pad:
+            raise ValueError(f"out_linearattn holds {B} x {vk_rows} rows; the GEMM has {M_pad} (tokens are padded to a multiple of 256 per batch entry)")
+        out = out_linearattn  # the q third is the plain store of this epilogue (epilogues.cuh:662-674)
+
     n_sc = max(1, math.ceil(rank_up / 16))
     sc = (ctypes.c_float * n_sc)(*[float(lora_scales[i]) if i < len(lora_scales) else 0.0 for i in range(n_sc)])
     M_out = 0 if out is None else out.numel() // out.shape[-1]
@@ -203,6 +230,7 @@ def svdq_gemm_w4a4(
         rot_rows=0 if rot_n is None else rot_n.shape[0], norm_eps=NORM_EPS, k_split=int(K_SPLIT or 0),
         out_q=nv.ptr(out_q), out_k=nv.ptr(out_k), out_v=nv.ptr(out_v), qkv_head_stride=(ctypes.c_int64 * 3)(*qkv_strides),
         attn_tokens=int(attn_tokens) if out_q is not None else 0, qkv_rows=M_pad if out_q is not None else 0,
+        out_vk=nv.ptr(out_vk), vk_rows=vk_rows,
     )
     with torch.cuda.device(dev):  # the library launches on the current device
         entry = nv.lib().svdq_gemm_w4a4_noalloc if NO_ALLOC else nv.lib().svdq_gemm_w4a4

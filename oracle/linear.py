@@ -193,3 +193,40 @@ def pack_qkv(out: torch.Tensor, attn_tokens: int) -> tuple[torch.Tensor, torch.T
         t[:, attn_tokens:, :] = mask
         parts.append(t[None])
     return tuple(parts)
+
+
+def litela(out: torch.Tensor, batch: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """EpilogueLiteLA (src/kernels/zgemm/epilogues.cuh:552-681) on the output of a fused QKV projection of a
+    linear-attention block, selected as in gemm_w4a4_launch_impl.cuh:311-345.
+
+    out fp32 [batch * tokens_pad, N], N = 3 * heads * 32, before the bf16 rounding of the GEMM tile.  Columns
+    [0, N/3) are q: ``relu`` (:662-664).  The other columns hold, per head, 32 of k then 32 of v (:600-603): with
+    k' = relu(k) (:605-607), ``vk[b, h, i, j] = sum_t v[t, i] * k'[t, j]`` for i < 32 (:598-622; row = v index,
+    column = k index) and ``vk[b, h, 32, j] = sum_t k'[t, j]`` (:624-646, v replaced by ones), over ALL rows of batch
+    entry b, padding rows included, in fp32 on the bf16-rounded values.
+    Returns (q fp32 [batch, tokens_pad, N/3] holding bf16 values, vk fp64 [batch, heads, 33, 32]).
+    """
+    M, N = out.shape
+    assert N % 96 == 0 and M % batch == 0
+    heads, rows = N // 96, M // batch
+    x = out.to(torch.bfloat16).to(torch.float64)
+    q = torch.relu(x[:, : N // 3]).reshape(batch, rows, N // 3).to(torch.float32)
+    kv = x[:, N // 3:].reshape(batch, rows, heads, 64)
+    k, v = torch.relu(kv[..., :32]), kv[..., 32:]
+    vk = torch.zeros(batch, heads, 33, 32, dtype=torch.float64)
+    vk[:, :, :32] = torch.einsum("bthi,bthj->bhij", v, k)
+    vk[:, :, 32] = k.sum(dim=1)
+    return q, vk
+
+
+def linearattn_vk_mul_q(q: torch.Tensor, vk: torch.Tensor, num_tokens: int, eps: float = 1e-6) -> torch.Tensor:
+    """vk_mul_q_kernel (epilogues.cuh:683-744): per token and head, ``o[j] = sum_i q[i] * vk[j][i]`` for j <= 32,
+    result ``o[:32] / (o[32] + eps)``; rows from ``num_tokens`` on keep their input.  fp64; q [B, T, heads * 32],
+    vk [B, heads, 33, 32]."""
+    B, T, W = q.shape
+    heads = W // 32
+    qh = q.to(torch.float64).reshape(B, T, heads, 32)
+    o = torch.einsum("bthi,bhji->bthj", qh, vk.to(torch.float64))
+    res = (o[..., :32] / (o[..., 32:] + eps)).reshape(B, T, W)
+    res[:, num_tokens:] = q.to(torch.float64)[:, num_tokens:]
+    return res

@@ -173,7 +173,7 @@ def test_python_wrappers_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU"):
         svdq_quantize_w4a4_act_fuse_lora(x, lora_down=torch.zeros(128, 16, dtype=torch.bfloat16))
     with pytest.raises(NotImplementedError):
-        svdq_gemm_w4a4(act=x, wgt=x, out_vk=x)
+        svdq_gemm_w4a4(act=x, wgt=x, poolout=x)
     with pytest.raises(RuntimeError, match="GPU"):
         svdq_gemm_w4a4(act=x.view(torch.uint8), wgt=x.view(torch.int8), ascales=x, wscales=x, out=x)
 

@@ -179,3 +179,50 @@ def test_rows_are_independent_and_linear_in_the_weights():
     ones_a, ones_w = torch.ones(2, 4, dtype=torch.bfloat16), torch.ones(2, 8, dtype=torch.bfloat16)
     want = (codes.to(torch.int32) @ wq.to(torch.int32).t()).float()
     assert torch.equal(olin.gemm_w4a4(quant.dequant_int4(codes, ones_a), quant.dequant_int4(wq, ones_w)), want)
+
+
+def test_litela_literal_answers():
+    """One head (N = 96), two batch entries of two rows each.  Column order [q 32 | k 32 | v 32], the ReLU on q and
+    k but not on v, v index = row of vk and k index = column, the ones row, the batch split: all by hand."""
+    out = torch.zeros(4, 96)
+    # batch 0, row 0: q0 = -1 (ReLU -> 0), q1 = 2; k0 = 3, k1 = -5 (ReLU -> 0); v0 = -2, v3 = 0.5
+    out[0, 0], out[0, 1] = -1.0, 2.0
+    out[0, 32], out[0, 33] = 3.0, -5.0
+    out[0, 64], out[0, 67] = -2.0, 0.5
+    # batch 0, row 1: k0 = 1, k2 = 4; v0 = 10
+    out[1, 32], out[1, 34] = 1.0, 4.0
+    out[1, 64] = 10.0
+    # batch 1, row 0 (row 2 of the GEMM): k5 = 1.00390625 (bf16 tie -> 1.0), v7 = 7
+    out[2, 32 + 5] = 1.00390625
+    out[2, 64 + 7] = 7.0
+    q, vk = olin.litela(out, batch=2)
+    assert q.shape == (2, 2, 32) and vk.shape == (2, 1, 33, 32)
+    assert q[0, 0, 0] == 0.0 and q[0, 0, 1] == 2.0 and q.abs().sum() == 2.0
+    want = torch.zeros(33, 32, dtype=torch.float64)
+    want[0, 0] = -2.0 * 3.0 + 10.0 * 1.0   # v0 k0 over both rows = 4
+    want[0, 2] = 10.0 * 4.0                # v0 k2
+    want[3, 0] = 0.5 * 3.0                 # v3 k0
+    want[32, 0] = 3.0 + 1.0                # sums of relu(k)
+    want[32, 2] = 4.0
+    assert torch.equal(vk[0, 0], want)     # (k1 = -5 contributes nowhere: not to row 0, not to the sums)
+    want1 = torch.zeros(33, 32, dtype=torch.float64)
+    want1[7, 5] = 7.0
+    want1[32, 5] = 1.0
+    assert torch.equal(vk[1, 0], want1)
+
+
+def test_linearattn_vk_mul_q_literal_answers():
+    vk = torch.zeros(1, 2, 33, 32)
+    vk[0, 0, 0, 0], vk[0, 0, 0, 1] = 2.0, 1.0     # o[0] = 2 q0 + q1
+    vk[0, 0, 5, 1] = 3.0                          # o[5] = 3 q1
+    vk[0, 0, 32, 0], vk[0, 0, 32, 1] = 1.0, 1.0   # denominator q0 + q1
+    vk[0, 1, 1, 0] = 4.0                          # head 1: o[1] = 4 q0, denominator 0 + eps
+    q = torch.zeros(1, 3, 64)
+    q[0, 0, 0], q[0, 0, 1] = 1.0, 3.0             # head 0 of token 0
+    q[0, 0, 32] = 0.5                             # head 1 of token 0
+    q[0, 2, 0] = 9.0                              # token 2 is beyond num_tokens
+    got = olin.linearattn_vk_mul_q(q, vk, num_tokens=2, eps=0.25)
+    assert got[0, 0, 0].item() == 5.0 / 4.25 and got[0, 0, 5].item() == 9.0 / 4.25
+    assert got[0, 0, 33].item() == 2.0 / 0.25
+    assert got[0, 2, 0].item() == 9.0 and got[0, 1].abs().sum() == 0.0
+    assert got[0, 0].count_nonzero() == 3
