@@ -99,6 +99,18 @@ def test_mlp_flux_shape(dev):
                    lora_act_in=la, lora_up=t1["proj_up"], lora_down=t2["proj_down"], lora_act_out=la2, bias=t1["bias"],
                    smooth_factor=t2["smooth_factor"])
     torch.cuda.synchronize()
+    # The low-rank input of fc2 is summed over 48 column blocks by workgroups that finish in no fixed order: the sums
+    # are formed in fixed point, so a second launch must reproduce them, and with them the layer output, bit for bit.
+    la2_first, y_first = la2.clone(), y.clone()
+    for _ in range(3):
+        la2.fill_(float("nan"))
+        svdq_gemm_w4a4(act=qx, wgt=t1["qweight"], out=out, qout=qout, ascales=asc, wscales=t1["wscales"], oscales=osc,
+                       lora_act_in=la, lora_up=t1["proj_up"], lora_down=t2["proj_down"], lora_act_out=la2, bias=t1["bias"],
+                       smooth_factor=t2["smooth_factor"])
+        y_again = fused_gelu_mlp(x.to(dev).view(1, M, c1["K"]), m1, m2)[0]
+        torch.cuda.synchronize()
+        assert torch.equal(la2, la2_first), "the next layer's low-rank input changed between two launches"
+        assert torch.equal(y_again, y_first), "the fused MLP's output changed between two launches"
     rows = torch.randperm(M, generator=torch.Generator().manual_seed(3))[:128]
     h = out.cpu()[rows]
     want_codes, want_scales = quant.quantize_act_int4(h, fc2.smooth, unsigned=True, shift=quant.SHIFT_GELU)

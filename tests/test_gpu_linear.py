@@ -7,7 +7,7 @@ import torch
 
 from conftest import announce
 from gpu_util import check_output, make_module, make_oracle
-from oracle import synth
+from oracle import quant, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -93,6 +93,26 @@ def _full_shape_properties(dev, name, sample_rows=192, linearity=True):
     rows = torch.randperm(M, generator=torch.Generator().manual_seed(0))[:sample_rows]
     want = ref.forward_quant(codes[rows], scales[:, rows], lora[rows])
     check_output(y[rows], want)
+    # Every tile of the output, through two checksums: the sum of each row and the sum of each column, against the same
+    # sums of the oracle's formula taken before the matrix product (weights summed over the output channels, activations
+    # over the rows).  A tile that is missing, stale or from the wrong place moves 128 column sums or 256 row sums by
+    # about sqrt(128) .. sqrt(256) typical magnitudes; the bf16 rounding of the summed elements moves them by
+    # sqrt(count) * 2^-9 of one.
+    a = (quant.dequant_nvfp4(codes, scales) if fp4 else quant.dequant_int4(codes, scales))[:M].double()
+    w = ref.w_deq.double()
+    cf = torch.full((N,), float(ref.wtscale), dtype=torch.float64)
+    if ref.wcscales is not None:
+        cf = cf * ref.wcscales.double()
+    lora_b = lora[:M].to(torch.bfloat16).double()
+    up = layer.proj_up.double()
+    bias = layer.bias.double()
+    want_rows = a @ (w * cf[:, None]).sum(0) + bias.sum() + lora_b @ up.sum(0)
+    want_cols = cf * (w @ a.sum(0)) + M * bias + up @ lora_b.sum(0)
+    yd = y.double()
+    rms = yd.pow(2).mean().sqrt().item()
+    got_rows, got_cols = yd.sum(1).cpu(), yd.sum(0).cpu()
+    assert (got_rows - want_rows).abs().max().item() <= 6 * N**0.5 * 2.0**-9 * rms, "row checksums"
+    assert (got_cols - want_cols).abs().max().item() <= 6 * M**0.5 * 2.0**-9 * rms, "column checksums"
     if linearity:
         # bias linearity: y(bias) - y(0) == bias up to bf16 rounding of the two outputs
         m0 = make_module(synth.LogicalLayer(**{**layer.__dict__, "bias": torch.zeros_like(layer.bias)}), dev)
