@@ -78,7 +78,14 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
                              (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)xbase);
     const __amdgpu_buffer_rsrc_t xrsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)xbase_s, 0, __builtin_amdgcn_readfirstlane(rows_valid * ld * 2), RSRC_WORD3);
-    const uint32_t x_voff = (uint32_t)(r * ld + 32 * XW * q) * 2;
+    // A load instruction fetches whole 256-byte (512 with GLU) runs of consecutive rows, 16 bytes per lane: rows
+    // RPI * i + lane / PPR, 16-byte piece lane % PPR.  (Every cache line is then touched by one instruction only;
+    // fetching the matrix-core operand layout directly, 16 rows x 64 scattered bytes per instruction, was 15 % slower
+    // on the whole kernel.)  The pieces are brought into that layout through a per-wave LDS area, see below.
+    constexpr int PPR = 16 * XW, RPI = 64 / PPR;  // pieces per row, rows per instruction
+    const uint32_t x_voff = (uint32_t)((lane / PPR) * ld * 2 + (lane % PPR) * 16);
+    __shared__ __attribute__((aligned(16))) uint8_t transpose_area[NW][16 * PPR * 16];
+    uint8_t *tr = transpose_area[wave];
 
     // x of one chunk: MT tiles x 4 steps x 8 bf16 per lane (twice that with GLU)
     // Requests are unconditional (a request behind a branch makes the compiler's wait counting assume the
@@ -91,7 +98,7 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int i = 0; i < XL; i++)
-                xv[mt][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (x_voff | beyond) + (uint32_t)(16 * mt * ld) * 2 + 16 * i, c * 256 * XW, 0);
+                xv[mt][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (x_voff | beyond) + (uint32_t)((16 * mt + RPI * i) * ld) * 2, c * 256 * XW, 0);
     };
     // proj_down as a buffer too: empty when there is no low-rank branch, so that its requests need no branch
     const __amdgpu_buffer_rsrc_t drsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.down, 0, RT > 0 ? p.K * p.R * 2 : 0, RSRC_WORD3);
@@ -109,8 +116,23 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
         __syncthreads();
     }
 
-    auto process = [&](int c, u32x4_t (&xraw)[MT][XL], u32x4_t (&x_ahead)[MT][XL]) {
+    auto process = [&](int c, u32x4_t (&xin)[MT][XL], u32x4_t (&x_ahead)[MT][XL]) {
         const int kbase = 128 * c + 32 * q;
+        // ---- from the load layout to the operand layout: lane (r, q) gets the XL pieces XL * q + i of row r.
+        // Row-major in LDS with the pieces of row r rotated by r: the 16 lanes of a write (one row, 16 pieces)
+        // and the 16 lanes of a read (16 rows, one piece) then both hit 16 different bank groups.  The area is
+        // private to the wave, whose LDS operations complete in order.
+        u32x4_t xraw[MT][XL];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+            for (int i = 0; i < XL; i++) {
+                const int row = RPI * i + lane / PPR, piece = lane % PPR;
+                *(u32x4_t *)(tr + row * (PPR * 16) + ((piece + row) % PPR) * 16) = xin[mt][i];
+            }
+#pragma unroll
+            for (int i = 0; i < XL; i++) xraw[mt][i] = *(const u32x4_t *)(tr + r * (PPR * 16) + ((XL * q + i + r) % PPR) * 16);
+        }
         // ---- requests first: the low-rank operands of this chunk (all four steps when they fit the
         // registers), then the activations DEPTH chunks ahead.  In this order a wait for the operands
         // does not wait for the activations.
@@ -293,7 +315,7 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         if (RT <= 4) return launch<4, 1, 4, 1, FP4, true>(p, stream);
         if (RT <= 8) return launch<4, 1, 8, 1, FP4, true>(p, stream);
     } else {
-        if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4, false>(p, stream) : launch<4, 1, 2, 2, FP4, false>(p, stream);
+        if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4, false>(p, stream) : launch<4, 1, 2, 1, FP4, false>(p, stream);
         if (RT <= 4) return launch<4, 2, 4, 1, FP4, false>(p, stream);
         if (RT <= 8) return launch<4, 2, 8, 1, FP4, false>(p, stream);
     }

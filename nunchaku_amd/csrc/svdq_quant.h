@@ -76,16 +76,22 @@ __device__ inline void quantize_int4_half_group_e2m3(const float (&y)[32], int p
     typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
     float amax = 0.f;
 #pragma unroll
-    for (int e = 0; e < 32; e++) amax = fmaxf(amax, fabsf(y[e]));
+    for (int e = 0; e < 32; e += 2) amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fabsf(y[e])), __builtin_fabsf(y[e + 1]));  // one three-way maximum per pair
     amax = fmaxf(amax, __shfl_xor(amax, partner_xor));
     const float s = __fmul_rn(amax, UNSIGNED ? RECIP_15 : RECIP_7);
     const float rcp = s > 0.f ? __fdiv_rn(1.0f, s) : 0.f;
-    const float cl = UNSIGNED ? 0.0f : -8.0f, ch = UNSIGNED ? 15.0f : 7.0f;
     float16_t ev, od;
 #pragma unroll
     for (int e = 0; e < 16; e++) {
-        ev[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e], rcp), cl, ch));
-        od[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e + 1], rcp), cl, ch));
+        if (UNSIGNED) {
+            ev[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e], rcp), 0.0f, 15.0f));
+            od[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e + 1], rcp), 0.0f, 15.0f));
+        } else {
+            // signed codes need no clamp: |y| <= amax and rcp = fl(1 / fl(amax / 7)) give |y * rcp| <= 7 (1 + 2^-21),
+            // which rounds to 7 at most (the reference clamps to [-8, 7], which these values never leave)
+            ev[e] = __builtin_rintf(__fmul_rn(y[2 * e], rcp));
+            od[e] = __builtin_rintf(__fmul_rn(y[2 * e + 1], rcp));
+        }
     }
     const u32x6_t w = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, 2.0f);
     lo = u32x4_t{w[0], w[1], w[2], w[3]};
