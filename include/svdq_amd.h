@@ -217,7 +217,7 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
  * until the process ends: 10 MB for arrival counters and fixed-point sums, 32 MB for partial sums) instead
  * of allocating one: no hipMalloc, hipFree or other allocating call is made.  A call whose need exceeds
  * the array returns SVDQ_EUNSUPPORTED with a message that says how much it wanted (examples that fit:
- * INT4 M_pad = 256, K = N = 3072 split six ways, 18.9 MB of partial sums; next_lora_down with M_pad * R_down
+ * INT4 M_pad = 256, K = N = 3072 split six ways (k_split = 6), 18.9 MB of partial sums; next_lora_down with M_pad * R_down
  * up to 1.3 M elements).  All calls on one GPU share the array, whatever their stream: calls that overlap
  * in time on one GPU race with each other.  What a launch needs to be zero at its start is cleared by a
  * fill kernel on `stream` first. */

@@ -196,18 +196,18 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     p.silu = a->fuse_silu != 0;
     p.gelu = a->qout != nullptr;  // the GELU is composed exactly when the next layer's input is produced (launch_impl.cuh:282-309)
 
-    // One workgroup per 128 x 256 output tile, two resident per compute unit.  With too few tiles to
-    // occupy the chip every tile is split along K into parts of at least 8 k-groups, whose partial sums
-    // meet in the workspace.
+    // One workgroup per 128 x 256 output tile, two resident per compute unit.  A tile alone on its compute
+    // unit takes about 30 us at K = 3072 whatever else the chip does, and every part of a split tile pays for
+    // parking its sums and the last one for fetching them all: measured at K = 3072, 24 tiles take 30.9 us
+    // whole, 28.3 in two parts, 36.1 in six, 106.7 in 24; 96 tiles 31.3 whole, 31.7 in two.  So only launches
+    // that fill at most an eighth of the slots are split, and only in two.
     const int mblocks = p.M_pad / g6::BM, nblocks = (p.N + g6::BN - 1) / g6::BN;
     const int ntiles = mblocks * nblocks, kgroups = p.K / 64, slots = 2 * ncu;
     int kparts = 1;
     if (a->k_split > 0) {
         kparts = a->k_split < kgroups ? a->k_split : kgroups;
-    } else if (2 * ntiles <= slots) {
-        kparts = slots / ntiles;
-        if (kparts > kgroups / 8) kparts = kgroups / 8;
-        if (kparts < 1) kparts = 1;
+    } else if (8 * ntiles <= slots && kgroups >= 16) {
+        kparts = 2;
     }
     p.kparts = kparts;
     const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu || a->out_vk != nullptr;
