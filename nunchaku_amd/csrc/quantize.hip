@@ -47,13 +47,22 @@ constexpr uint32_t RSRC_WORD3 = 0x00020000;  // raw buffer, 32-bit data format
 // and projected are bf16(value * bf16(gate * sigmoid(gate))) (load_act_to_fpsum<fuse_glu>,
 // gemm_base.cuh:612-623; silu, gemm_utils.cuh:322-327).  A lane then reads 64 consecutive input columns
 // for its 32, and everything after the product is as without GLU.
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU>
+//
+// ROWS (high ranks): the waves of a workgroup split its rows instead of its chunks: wave w owns the 16 MT rows
+// after row 16 MT (NW b + w) and all waves walk every chunk together.  The chunk of proj_down they all need (4 KB
+// per rank tile: 32 KB at rank 128, more than the activations of the chunk) is then fetched once per workgroup and
+// chunk, one chunk ahead, into an LDS double buffer; with chunks split among the waves every wave fetched its own
+// chunks' operands from the L2, one dependent request after the other.  No sums cross waves, so there is no
+// reduction at the end either.
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS>
 __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams p) {
-    extern __shared__ float lds[];  // smoothing factors [K] during the walk, then [NW waves][MT][RT][64][4] partial projections
+    // smoothing factors [K] during the walk; then, chunks split: [NW waves][MT][RT][64][4] partial projections;
+    // rows split: behind the factors two buffers of [4 steps][RT][64 lanes] x 16 bytes of proj_down
+    extern __shared__ float lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, q = lane >> 4;
-    const int row0 = blockIdx.x * (16 * MT);
+    const int row0 = ROWS ? (blockIdx.x * NW + wave) * (16 * MT) : blockIdx.x * (16 * MT);
     const int kgroups = p.K / 64;
     const int RT = p.R / 16;
     const int nchunks = p.K / 128;
@@ -108,11 +117,40 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
 
     // DEPTH chunks are requested ahead of the one being worked on
     u32x4_t xv[DEPTH + 1][MT][XL];
+    constexpr int CSTEP = ROWS ? 1 : NW;  // distance between the chunks a wave works on
+    const int cfirst = ROWS ? 0 : wave;
 #pragma unroll
-    for (int s = 0; s < DEPTH; s++) load_x(wave + s * NW, xv[s]);
+    for (int s = 0; s < DEPTH; s++) load_x(cfirst + s * CSTEP, xv[s]);
 
     if (SMOOTH == 1) {
         for (int k = threadIdx.x * 4; k < p.K; k += 64 * NW * 4) *(float4_t *)&lds[k] = *(const float4_t *)(p.smooth_rcp + k);
+        __syncthreads();
+    }
+
+    // rows split: wave w fetches the 1 KB pieces w, w + NW, ... of a chunk's 4 RT KB of proj_down
+    uint8_t *down_lds = (uint8_t *)lds + (SMOOTH == 1 ? (size_t)p.K * 4 : 0);
+    const int down_chunk_bytes = 4 * RT * 1024;
+    constexpr int DPW = ROWS ? (4 * RT_MAX + NW - 1) / NW : 1;  // pieces per wave
+    u32x4_t dstage[DPW];
+    auto fetch_down = [&](int c) {
+        const uint32_t beyond = c < nchunks ? 0u : 0x80000000u;
+#pragma unroll
+        for (int j = 0; j < DPW; j++) {
+            const int piece = wave + j * NW;
+            dstage[j] = __builtin_amdgcn_raw_buffer_load_b128(drsrc, (uint32_t)(lane * 16) | beyond | (piece < 4 * RT ? 0u : 0x80000000u),
+                                                              c * down_chunk_bytes + (piece < 4 * RT ? piece : 0) * 1024, 0);
+        }
+    };
+    auto park_down = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < DPW; j++) {
+            const int piece = wave + j * NW;
+            if (piece < 4 * RT) *(u32x4_t *)(down_lds + buf * down_chunk_bytes + piece * 1024 + lane * 16) = dstage[j];
+        }
+    };
+    if (ROWS && RT > 0) {
+        fetch_down(0);
+        park_down(0);
         __syncthreads();
     }
 
@@ -136,15 +174,16 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
         // ---- requests first: the low-rank operands of this chunk (all four steps when they fit the
         // registers), then the activations DEPTH chunks ahead.  In this order a wait for the operands
         // does not wait for the activations.
-        constexpr bool DOWN_UPFRONT = RT_MAX <= 2;
+        constexpr bool DOWN_UPFRONT = !ROWS && RT_MAX <= 2;
         bf16x8_t dn[DOWN_UPFRONT ? 4 : 1][RT_MAX];
+        if (ROWS) fetch_down(c + 1);
         if (DOWN_UPFRONT) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int rt = 0; rt < RT_MAX; rt++) dn[i][rt] = load_down(c, i, rt);
         }
-        load_x(c + DEPTH * NW, x_ahead);
+        load_x(c + DEPTH * CSTEP, x_ahead);
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- the gated unit: 16 (value, gate) pairs of two loads become the 8 bf16 of one step
@@ -241,24 +280,44 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int rt = 0; rt < RT_MAX; rt++) {
-                const bf16x8_t b = DOWN_UPFRONT ? dn[i][rt] : load_down(c, i, rt);
+                bf16x8_t b;
+                if (ROWS) b = *(const bf16x8_t *)(down_lds + (c & 1) * down_chunk_bytes + ((i * RT + (rt < RT ? rt : 0)) * 64 + lane) * 16);
+                else b = DOWN_UPFRONT ? dn[i][rt] : load_down(c, i, rt);
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++)
                     acc[mt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xs(mt, i)), b, acc[mt][rt], 0, 0, 0);
             }
+        if (ROWS && RT > 0) {
+            // the next chunk's operands go to the other buffer, which everybody finished reading before the
+            // previous barrier
+            park_down((c + 1) & 1);
+            __syncthreads();
+        }
     };
 
     // wave w walks the chunks w, w + NW, ...; the ring of DEPTH + 1 register buffers is indexed statically
-    for (int c0 = wave;; c0 += (DEPTH + 1) * NW) {
+    for (int c0 = cfirst;; c0 += (DEPTH + 1) * CSTEP) {
 #pragma unroll
         for (int s = 0; s <= DEPTH; s++) {
-            const int c = c0 + s * NW;
+            const int c = c0 + s * CSTEP;
             if (c >= nchunks) goto walked;
             process(c, xv[s], xv[(s + DEPTH) % (DEPTH + 1)]);
         }
     }
 walked:
 
+    if (ROWS) {
+        // every wave holds the finished sums of its own rows: lane l has rows 4 (l / 16) + [0, 4), rank l % 16 of a tile
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int rt = 0; rt < RT_MAX; rt++)
+                if (rt < RT) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) p.lora_out[(size_t)(row0 + 16 * mt + 4 * q + i) * p.R + 16 * rt + r] = acc[mt][rt][i];
+                }
+        return;
+    }
     // ---- reduce the waves' partial projections and write lora_act[row][rank]
     if (RT > 0) {
         if (SMOOTH == 1) __syncthreads();  // the factors in LDS are not needed any more
@@ -283,24 +342,25 @@ walked:
 
 constexpr size_t SMOOTH_LDS_MAX = 64 * 1024;  // two workgroups of a compute unit must fit side by side
 
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS = false>
 int launch_as(const QuantParams &p, hipStream_t stream) {
     size_t smem = (size_t)NW * MT * (p.R / 16) * 64 * 4 * sizeof(float);
     if (SMOOTH == 1 && (size_t)p.K * 4 > smem) smem = (size_t)p.K * 4;
-    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH, GLU>;
+    if (ROWS) smem = (SMOOTH == 1 ? (size_t)p.K * 4 : 0) + 2 * (size_t)(p.R / 16) * 4096;
+    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH, GLU, ROWS>;
     if (smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "quantize: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(kern, dim3(p.M_pad / (16 * MT)), dim3(64 * NW), smem, stream, p);
+    hipLaunchKernelGGL(kern, dim3(p.M_pad / (16 * MT * (ROWS ? NW : 1))), dim3(64 * NW), smem, stream, p);
     return check_launch("quantize_w4a4_act_fuse_lora");
 }
 
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, bool GLU>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, bool GLU, bool ROWS = false>
 int launch(const QuantParams &p, hipStream_t stream) {
-    if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0, GLU>(p, stream);
-    if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1, GLU>(p, stream);
-    return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2, GLU>(p, stream);
+    if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0, GLU, ROWS>(p, stream);
+    if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1, GLU, ROWS>(p, stream);
+    return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2, GLU, ROWS>(p, stream);
 }
 
 template <bool FP4, bool GLU>
@@ -315,6 +375,11 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         if (RT <= 4) return launch<4, 1, 4, 1, FP4, true>(p, stream);
         if (RT <= 8) return launch<4, 1, 8, 1, FP4, true>(p, stream);
     } else {
+        // High ranks with enough rows to give every compute unit work: the waves split the rows and share each
+        // chunk of proj_down through LDS (M = 18432, K = 3072: rank 128 68 us against 122, rank 64 51 against 71;
+        // at M = 4608 the few large workgroups lose: 65 against 42).
+        if (RT > 4 && p.M_pad >= 128 * 128) return launch<4, 2, 8, 1, FP4, false, true>(p, stream);
+        if (RT > 2 && RT <= 4 && p.M_pad >= 256 * 64) return launch<4, 1, 4, 1, FP4, false, true>(p, stream);
         if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4, false>(p, stream) : launch<4, 1, 2, 1, FP4, false>(p, stream);
         if (RT <= 4) return launch<4, 2, 4, 1, FP4, false>(p, stream);
         if (RT <= 8) return launch<4, 2, 8, 1, FP4, false>(p, stream);

@@ -202,3 +202,30 @@ def test_fuse_glu_random_gates(dev, fp4):
     assert (la - want_la).abs().max().item() <= 1e-3 * want_la.abs().max().item()
     # and the padding rows stay zero
     assert (codes[M:] == 0).all() and (la[M:] == 0).all()
+
+
+@pytest.mark.parametrize("M,K,R,fp4,smooth", [(16500, 256, 64, False, True), (16500, 384, 128, False, True), (16384, 256, 128, True, True),
+                                              (16400, 256, 96, False, False), (16384, 16512, 112, False, True)])
+def test_high_rank_many_rows(dev, M, K, R, fp4, smooth):
+    """Ranks above 32 with at least 16384 padded rows take the variant in which the waves of a workgroup split its rows and
+    share proj_down through LDS: ragged last workgroup (M = 16500: waves with some, and with no, valid rows), ranks that do
+    not fill the last rank tile pair (96, 112), NVFP4, no smoothing, K beyond what LDS holds of smoothing factors.  The
+    oracle runs on a sample of the rows (they are independent), all padding rows are checked to be zero."""
+    announce(f"quantize high rank M={M} K={K} R={R} fp4={fp4} smooth={smooth}")
+    layer = synth.make_layer(128, K, R, seed=R + K, fp4=fp4)
+    x = synth.make_activations(M, K, seed=M % 1000 + K)
+    codes, osc, la = _run(dev, x, layer, fp4=fp4, smooth=smooth)
+    M_pad = codes.shape[0]
+    g = torch.Generator().manual_seed(1)
+    rows = torch.cat([torch.arange(0, 130), torch.randperm(M, generator=g)[:190], torch.arange(M - 70, M)])
+    want_codes, want_scales, want_la = olin.quantize_act_fuse_lora(x[rows], layer.proj_down, layer.smooth if smooth else None, fp4=fp4)
+    n = rows.numel()
+    if fp4:
+        assert torch.equal(codes[rows].to(torch.uint8), want_codes[:n])
+        assert torch.equal(osc[:, rows].view(torch.uint8), want_scales[:, :n].view(torch.uint8))
+    else:
+        assert torch.equal(codes[rows], want_codes[:n])
+        assert torch.equal(osc[:, rows].view(torch.int16), want_scales[:, :n].view(torch.int16))
+    assert (la[rows] - want_la[:n]).abs().max().item() <= 2e-5 * want_la.abs().max().item() + 1e-6
+    assert (codes[M:] == 0).all() and (osc.float()[:, M:] == 0).all() and (la[M:] == 0).all()
+    assert not torch.isnan(la).any()
