@@ -130,8 +130,9 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * later call needs more (after a stream synchronisation), at most 16 pairs:
  *   - INT4 with so few output tiles that they are split along K (fewer tiles than compute units, or
  *     k_split > 1): 128 KB of fp32 partial sums per tile and part;
- *   - INT4 with next_lora_down: 8 bytes per element of next_lora_act_out (fixed-point sums, which make
- *     the result independent of the order in which the column blocks arrive);
+ *   - INT4 with next_lora_down: 4 bytes per element of next_lora_act_out and 256-column block of N (every
+ *     block leaves its share there and a small kernel launched behind the GEMM adds the shares in ascending
+ *     order, so the result does not depend on the order in which the blocks finish);
  *   - NVFP4 whenever the number of 256 x 256 tiles is not a multiple of the number of compute units:
  *     512 KB per compute unit.
  * Calls on one stream run in order and share the workspace safely; the same stream must not be used
@@ -214,11 +215,11 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
  * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  It runs the
  * same kernels as svdq_gemm_w4a4 and gives the same results bit for bit, but calls that need a workspace
  * (see above) take it from a fixed array in device memory (42 MB on every GPU the library runs on, held
- * until the process ends: 10 MB for arrival counters and fixed-point sums, 32 MB for partial sums) instead
+ * until the process ends: 10 MB for arrival counters, 32 MB for partial sums and low-rank shares) instead
  * of allocating one: no hipMalloc, hipFree or other allocating call is made.  A call whose need exceeds
  * the array returns SVDQ_EUNSUPPORTED with a message that says how much it wanted (examples that fit:
- * INT4 M_pad = 256, K = N = 3072 split six ways (k_split = 6), 18.9 MB of partial sums; next_lora_down with M_pad * R_down
- * up to 1.3 M elements).  All calls on one GPU share the array, whatever their stream: calls that overlap
+ * INT4 M_pad = 256, K = N = 3072 split six ways (k_split = 6), 18.9 MB of partial sums; next_lora_down at
+ * M_pad = 4608, N = 12288, R_down = 32, 28.3 MB of shares).  All calls on one GPU share the array, whatever their stream: calls that overlap
  * in time on one GPU race with each other.  What a launch needs to be zero at its start is cleared by a
  * fill kernel on `stream` first. */
 int svdq_gemm_w4a4_noalloc(const svdq_gemm_args *args, void *stream);

@@ -19,9 +19,9 @@ int launch_next(const Params &p, int nwg, hipStream_t stream);
 namespace {
 // Workspace of one (device, stream) pair: launches on one stream run one after the other and can share
 // it, launches on different streams may overlap and must not.  It is allocated the first time a launch
-// needs one and kept until the process ends.  The first `zero_bytes` hold arrival counters and
-// fixed-point sums: zero when allocated, and every launch that completes leaves them at zero again.
-// The rest is scratch (parked partial sums).
+// needs one and kept until the process ends.  The first `zero_bytes` hold arrival counters: zero when
+// allocated, and every launch that completes leaves them at zero again.  The rest is scratch (parked
+// partial sums, low-rank shares).
 struct Workspace {
     int dev;
     hipStream_t stream;
@@ -40,9 +40,36 @@ __global__ void zero_f32_kernel(float *p, int64_t n) {
     else for (int64_t j = i; j < n; j++) p[j] = 0.f;
 }
 
+// Sums the shares that the column blocks of a GEMM launch left for the next layer's low-rank projection
+// (gemm6_kernel.h, slot layout [column block][row block][row half][slab][rank tile][m2][64 lanes] x float4 with
+// lane l = rows 4 (l / 16) + [0, 4), rank l % 16 of a 16 x 16 tile) and writes lora_act [M_pad][R] row-major.
+__global__ void __launch_bounds__(256) reduce_shares_kernel(const float4_t *part, float *out, int nblocks, int mblocks, int R) {
+    const int quads_per_block = g6::BM * R / 4, RT = R / 16;
+    const int gq = blockIdx.x * 256 + threadIdx.x;
+    if (gq >= mblocks * quads_per_block) return;
+    const int mb = gq / quads_per_block, item = gq - mb * quads_per_block;
+    float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int b0 = 0; b0 < nblocks; b0 += 8) {  // eight requests in flight
+        float4_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = part[((size_t)(b0 + u < nblocks ? b0 + u : nblocks - 1) * mblocks + mb) * quads_per_block + item];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (b0 + u < nblocks) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) sum[e] += v[u][e];
+            }
+    }
+    const int ln = item & 63, m2 = (item >> 6) & 1, rest = item >> 7;  // rest = (row half * 2 + slab) * RT + rank tile
+    const int rt = rest % RT, slab32 = rest / RT;
+    const int row = mb * g6::BM + slab32 * 32 + 16 * m2 + 4 * (ln >> 4), rank = 16 * rt + (ln & 15);
+#pragma unroll
+    for (int e = 0; e < 4; e++) out[(size_t)(row + e) * R + rank] = sum[e];
+}
+
 void clear_zero_region(Workspace *w) {
     const int64_t n = (int64_t)(w->zero_bytes / 4);
-    hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, w->stream, (float *)w->ptr, n);
+    if (n > 0) hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, w->stream, (float *)w->ptr, n);
     w->dirty = false;
 }
 
@@ -88,7 +115,7 @@ Workspace *get_workspace(int dev, hipStream_t stream, size_t zero_bytes, size_t 
 
 // ---- the scratch of svdq_gemm_w4a4_noalloc --------------------------------------------------------
 // A fixed array in device memory, one copy per GPU, held until the process ends: first the region that
-// must be zero when a launch starts (arrival counters, fixed-point sums), then parked partial sums.
+// must be zero when a launch starts (arrival counters), then parked partial sums and low-rank shares.
 constexpr size_t NOALLOC_ZERO_BYTES = 10u << 20, NOALLOC_SCRATCH_BYTES = 32u << 20;
 static __device__ __align__(256) unsigned char scratch[NOALLOC_ZERO_BYTES + NOALLOC_SCRATCH_BYTES];
 uint8_t *g_scratch_ptr[64] = {nullptr};  // the array's device address on each GPU, asked once per GPU
@@ -174,8 +201,7 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     p.next_smooth_rcp = a->next_smooth_rcp;
     p.next_down = (const bf16x8_t *)a->next_lora_down;
     p.next_lora_out = a->next_lora_act_out;
-    p.next_lora_fix = nullptr;
-    p.next_lora_cnt = nullptr;
+    p.next_lora_part = nullptr;
     p.partials = nullptr;
     p.counters = nullptr;
     p.M_pad = (int)a->M_pad; p.N = (int)a->N; p.K = (int)a->K;
@@ -216,20 +242,26 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
         const size_t n = (size_t)(p.M_pad / p.vk_rows) * (p.N / 3 * 2 / 64) * g6::VK_HEAD_FLOATS;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, p.vk, (int64_t)n);
     }
-    const size_t cnt_bytes = (size_t)ntiles * 4, lcnt_bytes = (size_t)mblocks * 4;
-    const size_t fix_bytes = p.next_down ? (size_t)p.M_pad * p.R_down * 8 : 0;
+    const size_t cnt_bytes = (size_t)ntiles * 4;
     const size_t part_bytes = kparts > 1 ? (size_t)ntiles * kparts * g6::BM * g6::BN * 4 : 0;
+    const size_t share_bytes = p.next_down ? (size_t)nblocks * p.M_pad * p.R_down * 4 : 0;  // every column block's share of the next projection
     if (kparts == 1 && !p.next_down) return next ? g6::launch_next(p, ntiles, st) : g6::launch_plain(p, ntiles, st);
     std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
     if (!noalloc) lock.lock();
-    const size_t cnt_pad = (cnt_bytes + lcnt_bytes + 255) & ~(size_t)255;
+    const size_t cnt_pad = kparts > 1 ? (cnt_bytes + 255) & ~(size_t)255 : 0;
     WorkspaceView w;
-    if (!acquire_workspace(noalloc, dev, st, cnt_pad + fix_bytes, part_bytes, &w)) return noalloc && (cnt_pad + fix_bytes > NOALLOC_ZERO_BYTES || part_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
+    if (!acquire_workspace(noalloc, dev, st, cnt_pad, part_bytes + share_bytes, &w)) return noalloc && (cnt_pad > NOALLOC_ZERO_BYTES || part_bytes + share_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
     p.counters = (int *)w.zero;
-    p.next_lora_cnt = (int *)(w.zero + cnt_bytes);
-    p.next_lora_fix = (long long *)(w.zero + cnt_pad);
     p.partials = (float *)w.scratch;
-    const int rc = next ? g6::launch_next(p, ntiles * kparts, st) : g6::launch_plain(p, ntiles * kparts, st);
+    p.next_lora_part = (float *)(w.scratch + part_bytes);
+    int rc = next ? g6::launch_next(p, ntiles * kparts, st) : g6::launch_plain(p, ntiles * kparts, st);
+    if (rc == SVDQ_OK && p.next_down) {
+        // the column blocks' shares of the next layer's low-rank projection, added in ascending order
+        const int quads = p.M_pad * p.R_down / 4;
+        hipLaunchKernelGGL(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
+                           p.next_lora_out, nblocks, mblocks, p.R_down);
+        rc = check_launch("gemm_w4a4 (low-rank shares)");
+    }
     if (rc != SVDQ_OK && w.owner) w.owner->dirty = true;
     return rc;
 }

@@ -339,6 +339,16 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         if (ok && p.wcscales) cf *= bf16_bits_to_f32(p.wcscales[n]);
         coltab[tid] = cf;
         coltab[256 + tid] = (ok && p.bias) ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+        if (NEXT && p.next_down && p.R_down <= 32) {
+            // the next layer's proj_down for the tile's 256 columns (two 128-chunks, 4 KB per rank tile each,
+            // contiguous in memory) goes to LDS once: both row halves and both slabs read it from there
+            const int npieces = 8 * (p.R_down / 16);
+            for (int pc = wave; pc < npieces; pc += 4) {
+                if (n0 + (pc / (npieces / 2)) * 128 < p.N)
+                    *(u32x4_t *)(lds + EP_DOWN + pc * 1024 + lane * 16) =
+                        *(const u32x4_t *)((const uint8_t *)p.next_down + ((size_t)(n0 / 128) * (npieces / 2) + pc) * 1024 + lane * 16);
+            }
+        }
         if (NEXT && p.vk) {
             float *vkz = (float *)(lds + EP_VK);
             for (int i = tid; i < 2 * 2 * VK_HEAD_FLOATS; i += 256) vkz[i] = 0.f;
@@ -420,6 +430,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
             nrs[4 * i] = v4[0]; nrs[4 * i + 1] = v4[1]; nrs[4 * i + 2] = v4[2]; nrs[4 * i + 3] = v4[3];
         }
     }
+    const bool down_in_lds = NEXT && p.next_down && p.R_down <= 32;
     const bool interior = m0 + BM <= p.M_out && n0 + BN <= p.N_out;  // the whole tile lies inside the output
     uint16_t *slab = (uint16_t *)(lds + wave * SLAB_BYTES);
     const int ngroups_out = p.N / 64;
@@ -575,45 +586,63 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         }
         if (NEXT && p.next_down) {
             // Low-rank down projection of the next layer on the bf16 tile (EpilogueLoraDown,
-            // lora.cuh:243-353): this wave's 128 columns are one 128-chunk of the next layer's K.  The sums
-            // over the column blocks of all workgroups are formed with 64-bit integer atomics on fixed-point
-            // values (scale 2^32): integer addition is associative, so the result is the same from run to
-            // run whatever the order of arrival (the reference and fp32 atomics are not).  The two column
-            // halves of the workgroup meet in LDS first, which halves the number of atomics.
+            // lora.cuh:243-353): this wave's 128 columns are one 128-chunk of the next layer's K.  The two
+            // column halves of the workgroup meet in LDS (leaving that out and storing a share per half bought
+            // nothing); the sum goes to the workgroup's slot of the
+            // workspace, in the lanes' own order (a wave's store is 1 KB contiguous), and a small kernel launched
+            // behind this one adds the slots of all column blocks in ascending order (reduce_shares_kernel in
+            // gemm.hip): the same result from run to run, and this kernel never waits for its own stores.  (The
+            // reference adds with fp32 atomics in the order of arrival, lora.cuh:82-94.  Adding up inside this
+            // kernel, by whoever brings a row block's last share, needs every workgroup to wait until all its
+            // stores, the 64 KB of output included, have been acknowledged before it can say so: that wait cost
+            // 28 us at M = 4608, N = 12288, with atomics and with parked shares alike.)
             const int RT = p.R_down / 16;
             const int r16 = lane & 15, q = lane >> 4;
-            float *red = (float *)(lds + EP_RED);  // [row half][m2][64 lanes] x float4, reused by every rank tile
-            for (int rt = 0; rt < RT; rt++) {
-                float4_t d[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-                if (wcol0 < p.N) {
-                    bf16x8_t b[4];
+            float *red = (float *)(lds + EP_RED);  // [rank tile of the pair][row half][m2][64 lanes] x float4
+            const __amdgpu_buffer_rsrc_t slot = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(p.next_lora_part + ((size_t)nb * (p.M_pad / BM) + mb) * (size_t)(BM * p.R_down)), 0, BM * p.R_down * 4, 0x00020000);
+            for (int rt0 = 0; rt0 < RT; rt0 += 2) {
+                float4_t d[2][2];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) b[i] = p.next_down[((size_t)((wcol0 / 128) * 4 + i) * RT + rt) * 64 + lane];
+                for (int g = 0; g < 2; g++) {
+                    d[g][0] = d[g][1] = float4_t{0.f, 0.f, 0.f, 0.f};
+                    const int rt = rt0 + g;
+                    if (rt < RT && wcol0 < p.N) {
+                        bf16x8_t b[4];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
+                        for (int i = 0; i < 4; i++) {
+                            if (down_in_lds) b[i] = *(const bf16x8_t *)(lds + EP_DOWN + (((wn * 4 + i) * RT + rt) * 64 + lane) * 16);
+                            else b[i] = p.next_down[((size_t)((wcol0 / 128) * 4 + i) * RT + rt) * 64 + lane];
+                        }
 #pragma unroll
-                        for (int m2 = 0; m2 < 2; m2++) {
-                            const bf16x8_t a = *(const bf16x8_t *)(slab + (16 * m2 + r16) * OUT_LD + 32 * q + 8 * i);
-                            d[m2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[i], d[m2], 0, 0, 0);
+                        for (int i = 0; i < 4; i++) {
+#pragma unroll
+                            for (int m2 = 0; m2 < 2; m2++) {
+                                const bf16x8_t a = *(const bf16x8_t *)(slab + (16 * m2 + r16) * OUT_LD + 32 * q + 8 * i);
+                                d[g][m2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[i], d[g][m2], 0, 0, 0);
+                            }
                         }
                     }
                 }
                 if (wn == 1) {
 #pragma unroll
-                    for (int m2 = 0; m2 < 2; m2++) *(float4_t *)(red + ((wm * 2 + m2) * 64 + lane) * 4) = d[m2];
+                    for (int g = 0; g < 2; g++)
+#pragma unroll
+                        for (int m2 = 0; m2 < 2; m2++) *(float4_t *)(red + (((g * 2 + wm) * 2 + m2) * 64 + lane) * 4) = d[g][m2];
                 }
                 __syncthreads();
                 if (wn == 0) {
 #pragma unroll
-                    for (int m2 = 0; m2 < 2; m2++) {
-                        const float4_t o = *(const float4_t *)(red + ((wm * 2 + m2) * 64 + lane) * 4);
+                    for (int g = 0; g < 2; g++)
 #pragma unroll
-                        for (int i2 = 0; i2 < 4; i2++) {
-                            const long long fx = (long long)__builtin_rintf((d[m2][i2] + o[i2]) * 4294967296.0f);
-                            __hip_atomic_fetch_add(p.next_lora_fix + (size_t)(wrow0 + mt * 32 + 16 * m2 + 4 * q + i2) * p.R_down + 16 * rt + r16, fx,
-                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        for (int m2 = 0; m2 < 2; m2++) {
+                            if (rt0 + g >= RT) continue;
+                            const float4_t o = *(const float4_t *)(red + (((g * 2 + wm) * 2 + m2) * 64 + lane) * 4);
+                            const float4_t sum = float4_t{d[g][m2][0] + o[0], d[g][m2][1] + o[1], d[g][m2][2] + o[2], d[g][m2][3] + o[3]};
+                            // slot layout [row half wm][slab mt][rank tile][m2][64 lanes] x float4
+                            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), slot,
+                                                                   (((((wm * 2 + mt) * RT + rt0 + g) * 2 + m2) * 64) + lane) * 16, 0, 0);
                         }
-                    }
                 }
                 __syncthreads();
             }
@@ -672,28 +701,6 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
             if (col0 < third || col0 >= p.N) continue;
             const int head = (col0 - third) / 64 + rem / VK_HEAD_FLOATS;
             unsafeAtomicAdd(p.vk + ((size_t)batch * heads + head) * VK_HEAD_FLOATS + rem % VK_HEAD_FLOATS, vkall[i]);
-        }
-    }
-
-    if (NEXT && p.next_down) {
-        // The workgroup that adds the last column block's share to a block of 128 rows turns the
-        // fixed-point sums into fp32 and leaves sums and counter at zero for the next launch.
-        const int nblocks = (p.N + BN - 1) / BN;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this workgroup's atomics have been performed
-        __syncthreads();
-        int *flag = (int *)(lds + EP_FLAG);
-        if (tid == 0) *flag = __hip_atomic_fetch_add(p.next_lora_cnt + mb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        if (*flag == nblocks - 1) {
-            if (tid == 0) __hip_atomic_store(p.next_lora_cnt + mb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int n = BM * p.R_down;
-            long long *fix = p.next_lora_fix + (size_t)m0 * p.R_down;
-            float *dst = p.next_lora_out + (size_t)m0 * p.R_down;
-            for (int i = tid; i < n; i += 256) {
-                const long long s = __hip_atomic_load(fix + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(fix + i, 0ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                dst[i] = (float)((double)s * (1.0 / 4294967296.0));
-            }
         }
     }
 }

@@ -109,11 +109,14 @@ constexpr int SLAB_BYTES = 32 * OUT_LD * 2;
 constexpr int EP_TAB = 4 * SLAB_BYTES;     // float cf[256], bias[256]
 constexpr int EP_NORMW = EP_TAB + 2048;    // 4 waves x float [128]: RMS-norm weights of the wave's head
 constexpr int EP_FLAG = EP_NORMW + 2048;   // one word handed from thread 0 to the workgroup
-constexpr int EP_RED = EP_FLAG + 16;       // [2 row halves][2][64 lanes] x float4: the two column halves' low-rank sums meet here
-constexpr int EP_VK = EP_RED + 2 * 2 * 64 * 16;  // [2 column halves][2 heads][33][32] floats: linear-attention sums of the tile
+constexpr int EP_RED = EP_FLAG + 16;       // [2 rank tiles][2 row halves][2][64 lanes] x float4: the two column halves' low-rank sums meet here
+constexpr int EP_RED_BYTES = 2 * 2 * 2 * 64 * 16;  // two rank tiles at a time
+constexpr int EP_VK = EP_RED + EP_RED_BYTES;  // [2 column halves][2 heads][33][32] floats: linear-attention sums of the tile
+constexpr int EP_DOWN = EP_VK;                // or (never both): the next layer's proj_down for the tile's 256 columns, up to 2 rank tiles
 constexpr int VK_HEAD_FLOATS = 33 * 32;
-constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-static_assert(EP_VK + 2 * 2 * VK_HEAD_FLOATS * 4 <= LDS_BYTES, "the epilogue must fit the ring");
+constexpr int EP_END = EP_VK + 2 * 2 * VK_HEAD_FLOATS * 4;  // (the 16 KB of EP_DOWN are less)
+constexpr int LDS_BYTES = STAGES * STAGE_BYTES > EP_END ? STAGES * STAGE_BYTES : EP_END;
+static_assert(2 * LDS_BYTES <= 160 * 1024, "two workgroups share a compute unit's LDS");
 
 struct Params {
     const uint8_t *act;        // fragments [M_pad/128][K/64][4]
@@ -131,8 +134,7 @@ struct Params {
     const float *next_smooth_rcp;  // fp32 [N]
     const bf16x8_t *next_down;     // native proj_down of the next layer
     float *next_lora_out;          // fp32 [M_pad][R_down]
-    long long *next_lora_fix;      // [M_pad][R_down] fixed-point sums (zero between launches)
-    int *next_lora_cnt;            // [M_pad/128] arrival counters (zero between launches)
+    float *next_lora_part;         // [N/256 column blocks][M_pad/128][128 x R_down] partial projections, in the lanes' order
     // tiles split along K: parked partial sums and one arrival counter per tile (zero between launches)
     float *partials;
     int *counters;

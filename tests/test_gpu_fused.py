@@ -99,8 +99,9 @@ def test_mlp_flux_shape(dev):
                    lora_act_in=la, lora_up=t1["proj_up"], lora_down=t2["proj_down"], lora_act_out=la2, bias=t1["bias"],
                    smooth_factor=t2["smooth_factor"])
     torch.cuda.synchronize()
-    # The low-rank input of fc2 is summed over 48 column blocks by workgroups that finish in no fixed order: the sums
-    # are formed in fixed point, so a second launch must reproduce them, and with them the layer output, bit for bit.
+    # The low-rank input of fc2 is summed over 48 column blocks whose workgroups finish in no fixed order: the shares
+    # are added in ascending order afterwards, so a second launch must reproduce the sums, and with them the layer
+    # output, bit for bit.
     la2_first, y_first = la2.clone(), y.clone()
     for _ in range(3):
         la2.fill_(float("nan"))
