@@ -36,7 +36,7 @@ WORKLOADS = {
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, the peak the metric is quoted against
 # HBM-side bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
 # read for a device copy of known size (profiles/gemm6_kernel_*.md); only known for the profiled workload
-PROFILED_GEMM_TRAFFIC_BYTES = {"flux_mlp_fc1": (2.0 * 173320 + 1.0 * 110600) * 1024}
+PROFILED_GEMM_TRAFFIC_BYTES = {"flux_mlp_fc1": (2.0 * 144340 + 1.0 * 110590) * 1024}
 HBM_PEAK_GBS = 8000.0
 
 

@@ -236,6 +236,8 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
         kparts = 2;
     }
     p.kparts = kparts;
+    // bands of about ten row blocks, all of the same height where the count allows it
+    p.band = (mblocks + (mblocks + 9) / 10 - 1) / ((mblocks + 9) / 10);
     const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu || a->out_vk != nullptr;
     if (p.vk) {
         // the sums start at zero (the reference's launcher clears the tensor too, gemm_w4a4_launch_impl.cuh:335)

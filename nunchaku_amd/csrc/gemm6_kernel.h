@@ -105,16 +105,18 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
 
     // ---- which tile, which part of its k-groups ------------------------------------------------
     // Workgroups go to the XCDs round robin (blockIdx % 8); the remap gives each XCD one contiguous run
-    // of tile numbers, and the tiles are numbered in bands of 16 row blocks, down the band first: the 64
-    // workgroups resident on an XCD at one time then cover about 16 row blocks x 4 column blocks, whose
-    // operands (6 KB per row block and k-group, 14 KB per column block) they share in that XCD's L2.
+    // of tile numbers, and the tiles are numbered in bands of p.band row blocks (about ten), down the band
+    // first: the 64 workgroups resident on an XCD at one time then cover about 10 row blocks x 6 column
+    // blocks, whose operands (6 KB per row block and k-group, 14 KB per column block) they share in that
+    // XCD's L2.  Measured at 36 x 48 tiles, bytes fetched from beyond the L2 per launch: bands of 6 / 9 / 12 /
+    // 16 / 18 / 36 row blocks 317 / 296 / 308 / 355 / 396 / 604 MB (the time does not change: 169-171 us).
     const int mblocks = p.M_pad / BM, nblocks = (p.N + BN - 1) / BN;
     const int kgroups = p.K / 64;
     const int total = (int)gridDim.x;
     int v = (int)blockIdx.x;
     if (total % 8 == 0) v = (v % 8) * (total / 8) + v / 8;
     const int tile = v / p.kparts, part = v - tile * p.kparts;
-    constexpr int BAND = 16;
+    const int BAND = p.band;
     const int band = tile / (BAND * nblocks), in_band = tile - band * (BAND * nblocks);
     const int band_rows = mblocks - band * BAND < BAND ? mblocks - band * BAND : BAND;
     const int mb = band * BAND + in_band % band_rows, nb = in_band / band_rows;

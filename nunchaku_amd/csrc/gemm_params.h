@@ -138,6 +138,7 @@ struct Params {
     // tiles split along K: parked partial sums and one arrival counter per tile (zero between launches)
     float *partials;
     int *counters;
+    int band;          // row blocks per band of the tile numbering
     int kparts;
     int M_pad, N, K, M_out, N_out, R_up, R_down;
     float alpha;
