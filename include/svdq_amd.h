@@ -124,7 +124,7 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * INT4 runs on the fp6 matrix instruction (one workgroup per 128 x 256 output tile); NVFP4 runs on the
  * fp16 matrix instruction with dequantized operands (persistent workgroups, 256 x 256 tiles).
  *
- * Workspace.  Most INT4 calls need none and touch no global state.  Three kinds of call keep a
+ * Workspace.  Most INT4 calls need none and touch no global state.  Four kinds of call keep a
  * workspace per (device, stream) pair, allocated with hipMalloc the first time the pair needs it (that
  * call is not capturable into a graph and may synchronise), kept until the process ends, grown when a
  * later call needs more (after a stream synchronisation), at most 16 pairs:
@@ -133,6 +133,7 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  *   - INT4 with next_lora_down: 4 bytes per element of next_lora_act_out and 256-column block of N (every
  *     block leaves its share there and a small kernel launched behind the GEMM adds the shares in ascending
  *     order, so the result does not depend on the order in which the blocks finish);
+ *   - INT4 with out_vk: 4224 bytes per 32 rows and head;
  *   - NVFP4 whenever the number of 256 x 256 tiles is not a multiple of the number of compute units:
  *     512 KB per compute unit.
  * Calls on one stream run in order and share the workspace safely; the same stream must not be used
@@ -203,8 +204,9 @@ typedef struct svdq_gemm_args {
      *   out_vk[b][head][i][j] = sum over the vk_rows rows of batch entry b of v[row][i] * relu(k[row][j]),  i < 32,
      *   out_vk[b][head][32][j] = sum of relu(k[row][j]),
      * on the bf16-rounded values, accumulated in fp32.  Every row of the GEMM counts, padding rows included, as in
-     * the reference.  The library clears out_vk on `stream` first (the reference's launcher does, :335); sums of
-     * different row blocks arrive through fp32 atomics in no fixed order, as the reference's do (:649).       */
+     * the reference.  out_vk is fully written (the reference clears it first and adds with atomics in the order of
+     * arrival, :335, :649): every 32-row slab leaves its sums in the workspace and a small kernel launched behind the
+     * GEMM adds them in ascending order, so the result is the same from run to run.                             */
     float *out_vk;          /* fp32 [M_pad / vk_rows][2 N / 3 / 64][33][32]                                   */
     int64_t vk_rows;        /* rows per batch entry: a multiple of 256 that divides M_pad                     */
 } svdq_gemm_args;

@@ -67,6 +67,34 @@ __global__ void __launch_bounds__(256) reduce_shares_kernel(const float4_t *part
     for (int e = 0; e < 4; e++) out[(size_t)(row + e) * R + rank] = sum[e];
 }
 
+// Sums the linear-attention shares of the 32-row slabs of a GEMM launch (gemm6_kernel.h; per slab and head 1056 floats:
+// the 32 x 32 part [i][j] in the order of the matrix instruction's result registers, element e of lane l at
+// ((e / 4) * 64 + l) * 4 + e % 4 with i = 8 (e / 4) + 4 (l / 32) + e % 4, j = l % 32; then the 32 column sums) into
+// out_vk [batch][head][33][32].
+__global__ void __launch_bounds__(256) reduce_vk_kernel(const float *part, float *out, int batch, int slabs_per_batch, int heads) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= batch * heads * g6::VK_HEAD_FLOATS) return;
+    const int pos = idx % g6::VK_HEAD_FLOATS, head = (idx / g6::VK_HEAD_FLOATS) % heads, b = idx / (g6::VK_HEAD_FLOATS * heads);
+    int src = pos;  // row 32: stored as it is
+    if (pos < 1024) {
+        const int i = pos >> 5, j = pos & 31;
+        const int g = i >> 3, kb = (i >> 2) & 1, e3 = i & 3;
+        src = (g * 64 + kb * 32 + j) * 4 + e3;
+    }
+    const float *p0 = part + ((size_t)b * slabs_per_batch * heads + head) * g6::VK_HEAD_FLOATS + src;
+    const size_t stride = (size_t)heads * g6::VK_HEAD_FLOATS;
+    float sum = 0.f;
+    for (int s0 = 0; s0 < slabs_per_batch; s0 += 8) {  // eight requests in flight
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = p0[(size_t)(s0 + u < slabs_per_batch ? s0 + u : slabs_per_batch - 1) * stride];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (s0 + u < slabs_per_batch) sum += v[u];
+    }
+    out[idx] = sum;
+}
+
 void clear_zero_region(Workspace *w) {
     const int64_t n = (int64_t)(w->zero_bytes / 4);
     if (n > 0) hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, w->stream, (float *)w->ptr, n);
@@ -239,23 +267,21 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     // bands of about ten row blocks, all of the same height where the count allows it
     p.band = (mblocks + (mblocks + 9) / 10 - 1) / ((mblocks + 9) / 10);
     const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu || a->out_vk != nullptr;
-    if (p.vk) {
-        // the sums start at zero (the reference's launcher clears the tensor too, gemm_w4a4_launch_impl.cuh:335)
-        const size_t n = (size_t)(p.M_pad / p.vk_rows) * (p.N / 3 * 2 / 64) * g6::VK_HEAD_FLOATS;
-        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, p.vk, (int64_t)n);
-    }
     const size_t cnt_bytes = (size_t)ntiles * 4;
     const size_t part_bytes = kparts > 1 ? (size_t)ntiles * kparts * g6::BM * g6::BN * 4 : 0;
     const size_t share_bytes = p.next_down ? (size_t)nblocks * p.M_pad * p.R_down * 4 : 0;  // every column block's share of the next projection
-    if (kparts == 1 && !p.next_down) return next ? g6::launch_next(p, ntiles, st) : g6::launch_plain(p, ntiles, st);
+    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * g6::VK_HEAD_FLOATS * 4 : 0;  // every 32-row slab's linear-attention sums
+    if (kparts == 1 && !p.next_down && !p.vk) return next ? g6::launch_next(p, ntiles, st) : g6::launch_plain(p, ntiles, st);
     std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
     if (!noalloc) lock.lock();
     const size_t cnt_pad = kparts > 1 ? (cnt_bytes + 255) & ~(size_t)255 : 0;
     WorkspaceView w;
-    if (!acquire_workspace(noalloc, dev, st, cnt_pad, part_bytes + share_bytes, &w)) return noalloc && (cnt_pad > NOALLOC_ZERO_BYTES || part_bytes + share_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
+    const size_t scratch_bytes = part_bytes + share_bytes + vk_bytes;
+    if (!acquire_workspace(noalloc, dev, st, cnt_pad, scratch_bytes, &w)) return noalloc && (cnt_pad > NOALLOC_ZERO_BYTES || scratch_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
     p.counters = (int *)w.zero;
     p.partials = (float *)w.scratch;
     p.next_lora_part = (float *)(w.scratch + part_bytes);
+    p.vk_part = (float *)(w.scratch + part_bytes + share_bytes);
     int rc = next ? g6::launch_next(p, ntiles * kparts, st) : g6::launch_plain(p, ntiles * kparts, st);
     if (rc == SVDQ_OK && p.next_down) {
         // the column blocks' shares of the next layer's low-rank projection, added in ascending order
@@ -263,6 +289,13 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
         hipLaunchKernelGGL(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
                            p.next_lora_out, nblocks, mblocks, p.R_down);
         rc = check_launch("gemm_w4a4 (low-rank shares)");
+    }
+    if (rc == SVDQ_OK && p.vk) {
+        // the slabs' linear-attention sums, added per batch entry in ascending order of the rows
+        const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * g6::VK_HEAD_FLOATS;
+        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
+                           p.vk_rows / 32, heads);
+        rc = check_launch("gemm_w4a4 (linear-attention sums)");
     }
     if (rc != SVDQ_OK && w.owner) w.owner->dirty = true;
     return rc;

@@ -351,10 +351,6 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
                         *(const u32x4_t *)((const uint8_t *)p.next_down + ((size_t)(n0 / 128) * (npieces / 2) + pc) * 1024 + lane * 16);
             }
         }
-        if (NEXT && p.vk) {
-            float *vkz = (float *)(lds + EP_VK);
-            for (int i = tid; i < 2 * 2 * VK_HEAD_FLOATS; i += 256) vkz[i] = 0.f;
-        }
         if (NEXT && p.rotary && tid < 128) {
             // RMS-norm weights of the heads the two column halves are (q below N/3, k below 2N/3)
             ((float *)(lds + EP_NORMW))[tid] = bf16_bits_to_f32((n0 < p.rope_cols / 2 ? p.norm_q : p.norm_k)[tid]);
@@ -532,10 +528,13 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
             // EpilogueLiteLA::apply_litela (epilogues.cuh:572-655) on this slab: the wave's 128 columns are two
             // heads of [k 32 | v 32].  vk[i][j] = sum over the 32 rows of v[row][i] * relu(k[row][j]) on the
             // matrix cores (the rows are the contraction index: both operands are read down the columns of
-            // the slab), row 32 = sum of relu(k[row][j]).  The slabs and waves of the workgroup that share a
-            // head add up in LDS.
-            float *vkacc = (float *)(lds + EP_VK) + wn * (2 * VK_HEAD_FLOATS);
+            // the slab), row 32 = sum of relu(k[row][j]).  The slab's sums go to its own slot of the workspace
+            // ([32-row slab][head] x 1056 floats, the 32 x 32 part in the lanes' order: a wave's store is 1 KB
+            // contiguous); a small kernel behind this one adds the slabs of a batch entry in ascending order
+            // (reduce_vk_kernel in gemm.hip).  The reference adds with atomics in the order of arrival
+            // (epilogues.cuh:649); atomics here, 2.4 M of them at 4096 rows and 72 heads, doubled the kernel's time.
             const int j = lane & 31, kb = lane >> 5;
+            const int vheads = p.N / 3 * 2 / 64;
 #pragma unroll
             for (int hd = 0; hd < 2; hd++) {
                 float16_t d;
@@ -562,11 +561,11 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
                     d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vw), __builtin_bit_cast(bf16x8_t, kw), d, 0, 0, 0);
                 }
                 ks += __shfl_xor(ks, 32);
-                float *dst = vkacc + hd * VK_HEAD_FLOATS;
+                float *dst = p.vk_part + ((size_t)((wrow0 + mt * 32) >> 5) * vheads + (wcol0 - p.N / 3) / 64 + hd) * VK_HEAD_FLOATS;
 #pragma unroll
-                for (int e = 0; e < 16; e++)
-                    __hip_atomic_fetch_add(dst + ((e >> 2) * 8 + kb * 4 + (e & 3)) * 32 + j, d[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                if (kb == 0) __hip_atomic_fetch_add(dst + 32 * 32 + j, ks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                for (int g = 0; g < 4; g++)
+                    __builtin_nontemporal_store(float4_t{d[4 * g], d[4 * g + 1], d[4 * g + 2], d[4 * g + 3]}, (float4_t *)(dst + (g * 64 + lane) * 4));
+                if (kb == 0) dst[1024 + j] = ks;
             }
         }
         if (NEXT && p.qkv.q && wcol0 < p.N) store_qkv_slab(p.qkv, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N / 3);
@@ -690,21 +689,6 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     __builtin_amdgcn_sched_barrier(0);
     slab_epilogue(std::integral_constant<int, 0>{});
     slab_epilogue(std::integral_constant<int, 1>{});
-
-    if (NEXT && p.vk) {
-        // the tile's sums join those of the other row blocks (the reference's reduce_add, epilogues.cuh:649: the
-        // order of arrival decides the rounding there as here)
-        __syncthreads();
-        const float *vkall = (const float *)(lds + EP_VK);
-        const int third = p.N / 3, heads = 2 * third / 64, batch = m0 / p.vk_rows;
-        for (int i = tid; i < 2 * 2 * VK_HEAD_FLOATS; i += 256) {
-            const int half = i / (2 * VK_HEAD_FLOATS), rem = i - half * (2 * VK_HEAD_FLOATS);
-            const int col0 = n0 + half * 128;
-            if (col0 < third || col0 >= p.N) continue;
-            const int head = (col0 - third) / 64 + rem / VK_HEAD_FLOATS;
-            unsafeAtomicAdd(p.vk + ((size_t)batch * heads + head) * VK_HEAD_FLOATS + rem % VK_HEAD_FLOATS, vkall[i]);
-        }
-    }
 }
 
 template <bool NEXT>

@@ -111,10 +111,9 @@ constexpr int EP_NORMW = EP_TAB + 2048;    // 4 waves x float [128]: RMS-norm we
 constexpr int EP_FLAG = EP_NORMW + 2048;   // one word handed from thread 0 to the workgroup
 constexpr int EP_RED = EP_FLAG + 16;       // [2 rank tiles][2 row halves][2][64 lanes] x float4: the two column halves' low-rank sums meet here
 constexpr int EP_RED_BYTES = 2 * 2 * 2 * 64 * 16;  // two rank tiles at a time
-constexpr int EP_VK = EP_RED + EP_RED_BYTES;  // [2 column halves][2 heads][33][32] floats: linear-attention sums of the tile
-constexpr int EP_DOWN = EP_VK;                // or (never both): the next layer's proj_down for the tile's 256 columns, up to 2 rank tiles
+constexpr int EP_DOWN = EP_RED + EP_RED_BYTES;  // the next layer's proj_down for the tile's 256 columns, up to 2 rank tiles
 constexpr int VK_HEAD_FLOATS = 33 * 32;
-constexpr int EP_END = EP_VK + 2 * 2 * VK_HEAD_FLOATS * 4;  // (the 16 KB of EP_DOWN are less)
+constexpr int EP_END = EP_DOWN + 16384;
 constexpr int LDS_BYTES = STAGES * STAGE_BYTES > EP_END ? STAGES * STAGE_BYTES : EP_END;
 static_assert(2 * LDS_BYTES <= 160 * 1024, "two workgroups share a compute unit's LDS");
 
@@ -152,7 +151,8 @@ struct Params {
     // linear attention (EpilogueLiteLA, epilogues.cuh:552-681; next-layer variant only): columns [0, N/3) are q,
     // stored through `out` after a ReLU; the rest is [head][k 32 | v 32]; vk[batch][head][i][j] += sum over the
     // tile's rows of v[i] relu(k[j]) (i < 32) and of relu(k[j]) (i = 32)
-    float *vk;           // fp32 [batch][2 N / 3 / 64][33][32], zero before the launch; null: no such epilogue
+    float *vk;           // fp32 [batch][2 N / 3 / 64][33][32]; null: no such epilogue
+    float *vk_part;      // workspace: [M_pad / 32 slabs][heads] x 1056 floats, every slab's sums
     int vk_rows;         // rows per batch entry, a multiple of 256
 };
 }  // namespace g6
