@@ -130,10 +130,10 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * later call needs more (after a stream synchronisation), at most 16 pairs:
  *   - INT4 with so few output tiles that they are split along K (fewer tiles than compute units, or
  *     k_split > 1): 128 KB of fp32 partial sums per tile and part;
- *   - INT4 with next_lora_down: 4 bytes per element of next_lora_act_out and 256-column block of N (every
+ *   - next_lora_down: 4 bytes per element of next_lora_act_out and 256-column block of N (128 for NVFP4) (every
  *     block leaves its share there and a small kernel launched behind the GEMM adds the shares in ascending
  *     order, so the result does not depend on the order in which the blocks finish);
- *   - INT4 with out_vk: 4224 bytes per 32 rows and head;
+ *   - out_vk: 4224 bytes per 32 rows and head;
  *   - NVFP4 whenever the number of 256 x 256 tiles is not a multiple of the number of compute units:
  *     512 KB per compute unit.
  * Calls on one stream run in order and share the workspace safely; the same stream must not be used
@@ -197,7 +197,7 @@ typedef struct svdq_gemm_args {
     int64_t qkv_head_stride[3];
     int64_t attn_tokens;    /* rows that hold tokens (the reference's actualM of this epilogue)              */
     int64_t qkv_rows;       /* rows written per head, attn_tokens <= qkv_rows <= M_pad                       */
-    /* Linear attention (INT4 only; NULL / 0 otherwise).  Replaces EpilogueLiteLA,
+    /* Linear attention (NULL / 0 otherwise).  Replaces EpilogueLiteLA,
      * src/kernels/zgemm/epilogues.cuh:552-681, selected as in gemm_w4a4_launch_impl.cuh:311-345 (with `out` alone,
      * after bias and low-rank up).  N = 3 * heads * 32.  Columns [0, N/3) are q: `out` = bf16 [M_pad, N/3] receives
      * relu(q) (the reference's out_linearattn).  The other columns hold, per head, 32 of k then 32 of v, and

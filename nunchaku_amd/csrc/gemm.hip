@@ -40,29 +40,29 @@ __global__ void zero_f32_kernel(float *p, int64_t n) {
     else for (int64_t j = i; j < n; j++) p[j] = 0.f;
 }
 
-// Sums the shares that the column blocks of a GEMM launch left for the next layer's low-rank projection
-// (gemm6_kernel.h, slot layout [column block][row block][row half][slab][rank tile][m2][64 lanes] x float4 with
-// lane l = rows 4 (l / 16) + [0, 4), rank l % 16 of a 16 x 16 tile) and writes lora_act [M_pad][R] row-major.
-__global__ void __launch_bounds__(256) reduce_shares_kernel(const float4_t *part, float *out, int nblocks, int mblocks, int R) {
-    const int quads_per_block = g6::BM * R / 4, RT = R / 16;
-    const int gq = blockIdx.x * 256 + threadIdx.x;
-    if (gq >= mblocks * quads_per_block) return;
-    const int mb = gq / quads_per_block, item = gq - mb * quads_per_block;
+// Sums the shares that the column blocks (INT4 kernel: 256 columns each) or chunks (NVFP4 kernel: 128 columns) of a
+// GEMM launch left for the next layer's low-rank projection, in ascending order, and writes lora_act [M_pad][R]
+// row-major.  A share is [M_pad / 32 slabs][R / 16 rank tiles][2 halves of 16 rows][64 lanes] x float4, lane l holding
+// rows 4 (l / 16) + [0, 4), rank l % 16 of a 16 x 16 tile (the result registers of the matrix instruction).
+__global__ void __launch_bounds__(256) reduce_shares_kernel(const float4_t *part, float *out, int nshares, int M_pad, int R) {
+    const int RT = R / 16, quads = M_pad * R / 4;
+    const int item = blockIdx.x * 256 + threadIdx.x;
+    if (item >= quads) return;
     float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
-    for (int b0 = 0; b0 < nblocks; b0 += 8) {  // eight requests in flight
+    for (int b0 = 0; b0 < nshares; b0 += 8) {  // eight requests in flight
         float4_t v[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = part[((size_t)(b0 + u < nblocks ? b0 + u : nblocks - 1) * mblocks + mb) * quads_per_block + item];
+        for (int u = 0; u < 8; u++) v[u] = part[(size_t)(b0 + u < nshares ? b0 + u : nshares - 1) * quads + item];
 #pragma unroll
         for (int u = 0; u < 8; u++)
-            if (b0 + u < nblocks) {
+            if (b0 + u < nshares) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) sum[e] += v[u][e];
             }
     }
-    const int ln = item & 63, m2 = (item >> 6) & 1, rest = item >> 7;  // rest = (row half * 2 + slab) * RT + rank tile
+    const int ln = item & 63, m2 = (item >> 6) & 1, rest = item >> 7;  // rest = slab * RT + rank tile
     const int rt = rest % RT, slab32 = rest / RT;
-    const int row = mb * g6::BM + slab32 * 32 + 16 * m2 + 4 * (ln >> 4), rank = 16 * rt + (ln & 15);
+    const int row = slab32 * 32 + 16 * m2 + 4 * (ln >> 4), rank = 16 * rt + (ln & 15);
 #pragma unroll
     for (int e = 0; e < 4; e++) out[(size_t)(row + e) * R + rank] = sum[e];
 }
@@ -73,16 +73,16 @@ __global__ void __launch_bounds__(256) reduce_shares_kernel(const float4_t *part
 // out_vk [batch][head][33][32].
 __global__ void __launch_bounds__(256) reduce_vk_kernel(const float *part, float *out, int batch, int slabs_per_batch, int heads) {
     const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= batch * heads * g6::VK_HEAD_FLOATS) return;
-    const int pos = idx % g6::VK_HEAD_FLOATS, head = (idx / g6::VK_HEAD_FLOATS) % heads, b = idx / (g6::VK_HEAD_FLOATS * heads);
+    if (idx >= batch * heads * VK_HEAD_FLOATS) return;
+    const int pos = idx % VK_HEAD_FLOATS, head = (idx / VK_HEAD_FLOATS) % heads, b = idx / (VK_HEAD_FLOATS * heads);
     int src = pos;  // row 32: stored as it is
     if (pos < 1024) {
         const int i = pos >> 5, j = pos & 31;
         const int g = i >> 3, kb = (i >> 2) & 1, e3 = i & 3;
         src = (g * 64 + kb * 32 + j) * 4 + e3;
     }
-    const float *p0 = part + ((size_t)b * slabs_per_batch * heads + head) * g6::VK_HEAD_FLOATS + src;
-    const size_t stride = (size_t)heads * g6::VK_HEAD_FLOATS;
+    const float *p0 = part + ((size_t)b * slabs_per_batch * heads + head) * VK_HEAD_FLOATS + src;
+    const size_t stride = (size_t)heads * VK_HEAD_FLOATS;
     float sum = 0.f;
     for (int s0 = 0; s0 < slabs_per_batch; s0 += 8) {  // eight requests in flight
         float v[8];
@@ -270,7 +270,7 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     const size_t cnt_bytes = (size_t)ntiles * 4;
     const size_t part_bytes = kparts > 1 ? (size_t)ntiles * kparts * g6::BM * g6::BN * 4 : 0;
     const size_t share_bytes = p.next_down ? (size_t)nblocks * p.M_pad * p.R_down * 4 : 0;  // every column block's share of the next projection
-    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * g6::VK_HEAD_FLOATS * 4 : 0;  // every 32-row slab's linear-attention sums
+    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * VK_HEAD_FLOATS * 4 : 0;  // every 32-row slab's linear-attention sums
     if (kparts == 1 && !p.next_down && !p.vk) return next ? g6::launch_next(p, ntiles, st) : g6::launch_plain(p, ntiles, st);
     std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
     if (!noalloc) lock.lock();
@@ -287,12 +287,12 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
         // the column blocks' shares of the next layer's low-rank projection, added in ascending order
         const int quads = p.M_pad * p.R_down / 4;
         hipLaunchKernelGGL(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
-                           p.next_lora_out, nblocks, mblocks, p.R_down);
+                           p.next_lora_out, nblocks, p.M_pad, p.R_down);
         rc = check_launch("gemm_w4a4 (low-rank shares)");
     }
     if (rc == SVDQ_OK && p.vk) {
         // the slabs' linear-attention sums, added per batch entry in ascending order of the rows
-        const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * g6::VK_HEAD_FLOATS;
+        const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * VK_HEAD_FLOATS;
         hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
                            p.vk_rows / 32, heads);
         rc = check_launch("gemm_w4a4 (linear-attention sums)");
@@ -355,20 +355,41 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     p.partials = nullptr;
     p.counters = nullptr;
     // (the kernels with the next-layer epilogue also carry the norm + rotary epilogue)
-    const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu;
-    if (p.next_lora_out) {  // the low-rank projection for the next layer is accumulated across column blocks
-        const int64_t n = a->M_pad * a->R_down;
-        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, p.next_lora_out, n);
-    }
-    if (nwg <= ntiles && ntiles % nwg == 0) return next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
+    p.vk = a->out_vk;
+    p.vk_rows = (int)a->vk_rows;
+    p.vk_part = nullptr;
+    p.next_lora_part = nullptr;
+    const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu || a->out_vk != nullptr;
+    const bool shared_tiles = !(nwg <= ntiles && ntiles % nwg == 0);
+    // every 128-column chunk's share of the next layer's low-rank projection, every 32-row slab's linear-attention sums
+    const size_t share_bytes = p.next_down ? (size_t)(p.N / 128) * p.M_pad * p.R_down * 4 : 0;
+    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * VK_HEAD_FLOATS * 4 : 0;
+    if (!shared_tiles && !share_bytes && !vk_bytes) return next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
     std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
     if (!noalloc) lock.lock();
-    const size_t zero_bytes = (size_t)ntiles * 4, part_bytes = (size_t)2 * nwg * 256 * 64 * 16;
+    const size_t zero_bytes = shared_tiles ? (size_t)ntiles * 4 : 0, part_bytes = shared_tiles ? (size_t)2 * nwg * 256 * 64 * 16 : 0;
+    const size_t scratch_bytes = part_bytes + share_bytes + vk_bytes;
     WorkspaceView w;
-    if (!acquire_workspace(noalloc, dev, st, zero_bytes, part_bytes, &w)) return noalloc && (zero_bytes > NOALLOC_ZERO_BYTES || part_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
-    p.counters = (int *)w.zero;
-    p.partials = (float *)w.scratch;
-    const int rc = next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
+    if (!acquire_workspace(noalloc, dev, st, zero_bytes, scratch_bytes, &w)) return noalloc && (zero_bytes > NOALLOC_ZERO_BYTES || scratch_bytes > NOALLOC_SCRATCH_BYTES) ? SVDQ_EUNSUPPORTED : SVDQ_ELAUNCH;
+    if (shared_tiles) {
+        p.counters = (int *)w.zero;
+        p.partials = (float *)w.scratch;
+    }
+    p.next_lora_part = (float *)(w.scratch + part_bytes);
+    p.vk_part = (float *)(w.scratch + part_bytes + share_bytes);
+    int rc = next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
+    if (rc == SVDQ_OK && p.next_down) {
+        const int quads = p.M_pad * p.R_down / 4;
+        hipLaunchKernelGGL(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
+                           p.next_lora_out, p.N / 128, p.M_pad, p.R_down);
+        rc = check_launch("gemm_w4a4 (low-rank shares)");
+    }
+    if (rc == SVDQ_OK && p.vk) {
+        const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * VK_HEAD_FLOATS;
+        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
+                           p.vk_rows / 32, heads);
+        rc = check_launch("gemm_w4a4 (linear-attention sums)");
+    }
     if (rc != SVDQ_OK && w.owner) w.owner->dirty = true;
     return rc;
 }
@@ -399,7 +420,6 @@ int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
     }
     if (a->out_vk) {
         // EpilogueLiteLA (gemm_w4a4_launch_impl.cuh:311-345)
-        if (a->fp4) return fail(SVDQ_EUNSUPPORTED, "gemm: out_vk (linear attention) is built for INT4 operands only");
         SVDQ_REQUIRE(a->out && !a->qout && !a->rotary_emb && !a->next_lora_down && !a->fuse_silu, "gemm: out_vk goes with `out` (the q third) alone");
         SVDQ_REQUIRE(a->N % 384 == 0, "gemm: out_vk needs N (%lld) to be three equal parts of whole 128-column blocks", (long long)a->N);
         SVDQ_REQUIRE(a->vk_rows > 0 && a->vk_rows % 256 == 0 && a->M_pad % a->vk_rows == 0,

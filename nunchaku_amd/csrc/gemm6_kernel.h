@@ -524,50 +524,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         __builtin_amdgcn_wave_barrier();
         // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores.  Streaming stores: the
         // tile is not read again by this kernel.
-        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) {
-            // EpilogueLiteLA::apply_litela (epilogues.cuh:572-655) on this slab: the wave's 128 columns are two
-            // heads of [k 32 | v 32].  vk[i][j] = sum over the 32 rows of v[row][i] * relu(k[row][j]) on the
-            // matrix cores (the rows are the contraction index: both operands are read down the columns of
-            // the slab), row 32 = sum of relu(k[row][j]).  The slab's sums go to its own slot of the workspace
-            // ([32-row slab][head] x 1056 floats, the 32 x 32 part in the lanes' order: a wave's store is 1 KB
-            // contiguous); a small kernel behind this one adds the slabs of a batch entry in ascending order
-            // (reduce_vk_kernel in gemm.hip).  The reference adds with atomics in the order of arrival
-            // (epilogues.cuh:649); atomics here, 2.4 M of them at 4096 rows and 72 heads, doubled the kernel's time.
-            const int j = lane & 31, kb = lane >> 5;
-            const int vheads = p.N / 3 * 2 / 64;
-#pragma unroll
-            for (int hd = 0; hd < 2; hd++) {
-                float16_t d;
-#pragma unroll
-                for (int e = 0; e < 16; e++) d[e] = 0.f;
-                float ks = 0.f;
-#pragma unroll
-                for (int st = 0; st < 2; st++) {
-                    u32x4_t kw, vw;
-#pragma unroll
-                    for (int e = 0; e < 8; e += 2) {
-                        uint32_t kk[2], vv[2];
-#pragma unroll
-                        for (int f = 0; f < 2; f++) {
-                            const uint16_t *rowp = slab + (16 * st + 8 * kb + e + f) * OUT_LD + hd * 64 + j;
-                            kk[f] = rowp[0];
-                            vv[f] = rowp[32];
-                            if (kk[f] & 0x8000u) kk[f] = 0;  // ReLU on the bf16 value
-                            ks += bits_f32(kk[f] << 16);
-                        }
-                        kw[e / 2] = kk[0] | (kk[1] << 16);
-                        vw[e / 2] = vv[0] | (vv[1] << 16);
-                    }
-                    d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vw), __builtin_bit_cast(bf16x8_t, kw), d, 0, 0, 0);
-                }
-                ks += __shfl_xor(ks, 32);
-                float *dst = p.vk_part + ((size_t)((wrow0 + mt * 32) >> 5) * vheads + (wcol0 - p.N / 3) / 64 + hd) * VK_HEAD_FLOATS;
-#pragma unroll
-                for (int g = 0; g < 4; g++)
-                    __builtin_nontemporal_store(float4_t{d[4 * g], d[4 * g + 1], d[4 * g + 2], d[4 * g + 3]}, (float4_t *)(dst + (g * 64 + lane) * 4));
-                if (kb == 0) dst[1024 + j] = ks;
-            }
-        }
+        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) litela_slab(p.vk_part, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N);
         if (NEXT && p.qkv.q && wcol0 < p.N) store_qkv_slab(p.qkv, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N / 3);
         if (p.out && interior) {  // no bounds to check: all slab reads first, then all stores
             u32x4_t d[8];
@@ -640,7 +597,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
                             if (rt0 + g >= RT) continue;
                             const float4_t o = *(const float4_t *)(red + (((g * 2 + wm) * 2 + m2) * 64 + lane) * 4);
                             const float4_t sum = float4_t{d[g][m2][0] + o[0], d[g][m2][1] + o[1], d[g][m2][2] + o[2], d[g][m2][3] + o[3]};
-                            // slot layout [row half wm][slab mt][rank tile][m2][64 lanes] x float4
+                            // share layout [32-row slab][rank tile][m2][64 lanes] x float4; this workgroup's slabs are 4 mb + 2 wm + mt
                             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), slot,
                                                                    (((((wm * 2 + mt) * RT + rt0 + g) * 2 + m2) * 64) + lane) * 16, 0, 0);
                         }

@@ -706,6 +706,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #pragma unroll
                 for (int e = 0; e < 16; e++) v[nt][e] = gelu_tanh(v[nt][e]);
         }
+        if (NEXT && p.vk && wcol0 < p.N / 3) {
+            // the q third of a linear-attention projection is stored after a ReLU (epilogues.cuh:662-674)
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) v[nt][e] = __builtin_fmaxf(v[nt][e], 0.f);
+        }
         // bf16 tile -> per-wave LDS slab (32 rows x 128 columns), four columns per write: every later
         // consumer reads whole rows
 #pragma unroll
@@ -724,6 +731,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         __builtin_amdgcn_wave_barrier();
         // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores.  Streaming stores: the
         // tile is not read again by this kernel.
+        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) litela_slab(p.vk_part, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N);
         if (NEXT && p.qkv.q && wcol0 < p.N) store_qkv_slab(p.qkv, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N / 3);
         if (p.out && interior) {  // no bounds to check: all slab reads first, then all stores
             u32x4_t d[8];
@@ -767,11 +775,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                         d[m2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[i], d[m2], 0, 0, 0);
                     }
                 }
+                // This chunk's share of the sums over N goes to the workspace, in the lanes' own order; a small kernel
+                // behind this one adds the chunks' shares in ascending order (reduce_shares_kernel in gemm.hip): the
+                // same result from run to run (the reference adds with atomics in the order of arrival, lora.cuh:82-94).
 #pragma unroll
                 for (int m2 = 0; m2 < 2; m2++)
-#pragma unroll
-                    for (int i2 = 0; i2 < 4; i2++)
-                        atomicAdd(p.next_lora_out + (size_t)(wrow0 + mt * 32 + 16 * m2 + 4 * q + i2) * p.R_down + 16 * rt + r16, d[m2][i2]);
+                    __builtin_nontemporal_store(d[m2], (float4_t *)(p.next_lora_part + (size_t)(wcol0 / 128) * p.M_pad * p.R_down) +
+                                                           ((size_t)(((wrow0 + mt * 32) >> 5) * RT + rt) * 2 + m2) * 64 + lane);
             }
         }
         if (NEXT && p.qout && wcol0 < p.N) {

@@ -58,6 +58,52 @@ __device__ inline void store_qkv_slab(const QkvOut &o, const uint16_t *slab, int
     }
 }
 
+// Linear attention (EpilogueLiteLA::apply_litela, epilogues.cuh:572-655) on one 32-row x 128-column bf16 slab in LDS
+// (rows `ld` elements apart): the 128 columns are two heads of [k 32 | v 32].  vk[i][j] = sum over the 32 rows of
+// v[row][i] * relu(k[row][j]) on the matrix cores (the rows are the contraction index: both operands are read down
+// the columns of the slab), row 32 = sum of relu(k[row][j]).  The slab's sums go to its own slot of the workspace
+// ([32-row slab][head] x 1056 floats, the 32 x 32 part in the lanes' order: a wave's store is 1 KB contiguous); a
+// small kernel behind the GEMM adds the slabs of a batch entry in ascending order (reduce_vk_kernel in gemm.hip).
+// The reference adds with atomics in the order of arrival (epilogues.cuh:649); atomics here, 2.4 M of them at 4096
+// rows and 72 heads, doubled the kernel's time.
+constexpr int VK_HEAD_FLOATS = 33 * 32;
+__device__ inline void litela_slab(float *vk_part, const uint16_t *slab, int ld, int lane, int row0, int col0, int N) {
+    const int j = lane & 31, kb = lane >> 5;
+    const int vheads = N / 3 * 2 / 64;
+#pragma unroll
+    for (int hd = 0; hd < 2; hd++) {
+        float16_t d;
+#pragma unroll
+        for (int e = 0; e < 16; e++) d[e] = 0.f;
+        float ks = 0.f;
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            u32x4_t kw, vw;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                uint32_t kk[2], vv[2];
+#pragma unroll
+                for (int f = 0; f < 2; f++) {
+                    const uint16_t *rowp = slab + (16 * st + 8 * kb + e + f) * ld + hd * 64 + j;
+                    kk[f] = rowp[0];
+                    vv[f] = rowp[32];
+                    if (kk[f] & 0x8000u) kk[f] = 0;  // ReLU on the bf16 value
+                    ks += bits_f32(kk[f] << 16);
+                }
+                kw[e / 2] = kk[0] | (kk[1] << 16);
+                vw[e / 2] = vv[0] | (vv[1] << 16);
+            }
+            d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vw), __builtin_bit_cast(bf16x8_t, kw), d, 0, 0, 0);
+        }
+        ks += __shfl_xor(ks, 32);
+        float *dst = vk_part + ((size_t)(row0 >> 5) * vheads + (col0 - N / 3) / 64 + hd) * VK_HEAD_FLOATS;
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            __builtin_nontemporal_store(float4_t{d[4 * g], d[4 * g + 1], d[4 * g + 2], d[4 * g + 3]}, (float4_t *)(dst + (g * 64 + lane) * 4));
+        if (kb == 0) dst[1024 + j] = ks;
+    }
+}
+
 struct GemmParams {
     const uint8_t *act;
     const uint16_t *ascales;
@@ -90,6 +136,10 @@ struct GemmParams {
     int rot_rows, rope_cols;          // rope_cols = 2 N / 3: the columns of q and k
     float norm_eps;
     QkvOut qkv;
+    // linear attention (see g6::Params) and the parked shares of the next layer's low-rank projection
+    float *vk, *vk_part;
+    int vk_rows;
+    float *next_lora_part;  // [N/128 column chunks][M_pad/32 slabs][R_down/16][2][64 lanes] x float4
 };
 
 
@@ -112,7 +162,6 @@ constexpr int EP_FLAG = EP_NORMW + 2048;   // one word handed from thread 0 to t
 constexpr int EP_RED = EP_FLAG + 16;       // [2 rank tiles][2 row halves][2][64 lanes] x float4: the two column halves' low-rank sums meet here
 constexpr int EP_RED_BYTES = 2 * 2 * 2 * 64 * 16;  // two rank tiles at a time
 constexpr int EP_DOWN = EP_RED + EP_RED_BYTES;  // the next layer's proj_down for the tile's 256 columns, up to 2 rank tiles
-constexpr int VK_HEAD_FLOATS = 33 * 32;
 constexpr int EP_END = EP_DOWN + 16384;
 constexpr int LDS_BYTES = STAGES * STAGE_BYTES > EP_END ? STAGES * STAGE_BYTES : EP_END;
 static_assert(2 * LDS_BYTES <= 160 * 1024, "two workgroups share a compute unit's LDS");

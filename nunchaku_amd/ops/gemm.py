@@ -83,7 +83,7 @@ def svdq_gemm_w4a4(
     NaN (k) as in the reference (epilogues.cuh:427-550).  Within a head the values are plain [row, 128]; the
     reference orders them for its own attention kernel's matrix fragments.
     out_linearattn bf16 [B, tokens_pad, N/3] with out_vk fp32 [B, heads, 33, 32] (N = 3 * heads * 32, tokens_pad a
-    multiple of 256, INT4 only): linear attention (launch_impl.cuh:311-345): relu(q) goes to out_linearattn;
+    multiple of 256): linear attention (launch_impl.cuh:311-345): relu(q) goes to out_linearattn;
     out_vk[b, h, i, j] = sum over tokens of v[i] * relu(k[j]) (i < 32) and of relu(k[j]) (i = 32), where the
     columns after q hold, per head, 32 of k then 32 of v.  out_vk is cleared first.
     """
@@ -109,8 +109,6 @@ def svdq_gemm_w4a4(
     if out_vk is not None:
         if out is not None or qout is not None or out_q is not None or rotary_emb is not None or fuse_silu:
             raise ValueError("out_vk / out_linearattn go without out, qout, out_q and rotary_emb (launch_impl.cuh:282-417 picks one branch)")
-        if fp4:
-            raise NotImplementedError("the linear-attention epilogue is built for INT4 layers only")
     if out is None and qout is None and out_q is None and out_vk is None:
         raise ValueError("one of out / qout / (out_q, out_k, out_v) / (out_vk, out_linearattn) is required")
     if qout is not None and (oscales is None or smooth_factor is None):

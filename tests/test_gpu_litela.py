@@ -12,24 +12,30 @@ from oracle import synth
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("B,T,K,heads,R", [(1, 256, 256, 4, 16), (2, 256, 384, 8, 32), (1, 1024, 256, 12, 32), (3, 512, 128, 20, 0)])
-def test_litela_epilogue(dev, B, T, K, heads, R):
+@pytest.mark.parametrize("B,T,K,heads,R,fp4", [(1, 256, 256, 4, 16, False), (2, 256, 384, 8, 32, False), (1, 1024, 256, 12, 32, False),
+                                               (3, 512, 128, 20, 0, False), (2, 512, 256, 12, 32, True), (1, 2304, 128, 80, 16, True)])
+def test_litela_epilogue(dev, B, T, K, heads, R, fp4):
     """heads = 4: N = 384, one 256-column block of q + k/v and a ragged half block; 12 and 20 heads: the q third ends
     inside a 256-column block, so one workgroup holds a q half and a k/v half.  Several row blocks per batch entry add
-    up in a fixed order; several batch entries must not mix."""
+    up in a fixed order; several batch entries must not mix.  NVFP4: the other GEMM kernel (256 x 256 tiles; 2304 rows x
+    7680 columns are 270 tiles, which its workgroups share).  heads = 80: the q third ends inside a tile."""
     from nunchaku_amd.ops import svdq_gemm_w4a4
 
     N = heads * 96
-    announce(f"litela B={B} T={T} K={K} heads={heads} R={R}")
-    layer = synth.make_layer(N, K, R, seed=heads + K)
+    announce(f"litela B={B} T={T} K={K} heads={heads} R={R} fp4={fp4}")
+    layer = synth.make_layer(N, K, R, seed=heads + K, fp4=fp4)
     m = make_module(layer, dev)
     ref = make_oracle(layer)
+    if fp4:
+        ref.wtscale = float(torch.tensor(layer.wtscale).to(torch.bfloat16))  # the checkpoint stores wtscale as bf16
     x = synth.make_activations(B * T, K, seed=heads)
     qx, asc, la = m.quantize(x.to(dev))
     t = m.native_tensors()
     q = torch.full((B, T, N // 3), float("nan"), dtype=torch.bfloat16, device=dev)
     vk = torch.full((B, heads, 33, 32), float("nan"), dtype=torch.float32, device=dev)  # the operator clears it
     kw = dict(act=qx, wgt=t["qweight"], ascales=asc, wscales=t["wscales"], bias=t["bias"])
+    if fp4:
+        kw.update(fp4=True, alpha=m.alpha, wcscales=t["wcscales"])
     if R:
         kw.update(lora_act_in=la, lora_up=t["proj_up"])
     svdq_gemm_w4a4(**kw, out_vk=vk, out_linearattn=q)

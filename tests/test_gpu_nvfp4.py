@@ -63,13 +63,15 @@ def test_nvfp4_layer_end_to_end(dev):
     check_output(y, ref.forward_quant(codes, scales, lora)[:M])
 
 
-def test_nvfp4_fused_mlp_epilogue(dev):
-    """NVFP4 GEMM producing the next layer's NVFP4 input (no shift, signed patterns)."""
+@pytest.mark.parametrize("M,K1,N1,R", [(256, 256, 512, 16), (2304, 256, 7680, 32)])
+def test_nvfp4_fused_mlp_epilogue(dev, M, K1, N1, R):
+    """NVFP4 GEMM producing the next layer's NVFP4 input (no shift, signed patterns).  The second shape has 270 tiles,
+    which the persistent workgroups share, and 60 column chunks whose shares of the low-rank projection are added in
+    order afterwards: the projection must be fully written (it starts as NaN) and the same from launch to launch."""
     from nunchaku_amd import packing
     from nunchaku_amd.ops import svdq_gemm_w4a4
 
-    M, K1, N1, R = 256, 256, 512, 16
-    announce("nvfp4 next-layer epilogue")
+    announce(f"nvfp4 next-layer epilogue M={M} K1={K1} N1={N1} R={R}")
     fc1 = synth.make_layer(N1, K1, R, seed=41, fp4=True)
     fc2 = synth.make_layer(256, N1, R, seed=42, fp4=True)
     x = synth.make_activations(M, K1, seed=41)
@@ -79,11 +81,20 @@ def test_nvfp4_fused_mlp_epilogue(dev):
     out = torch.empty(M, N1, dtype=torch.bfloat16, device=dev)
     qout = torch.empty(M, N1 // 2, dtype=torch.uint8, device=dev)
     osc = torch.empty(N1 // 16, M, dtype=torch.float8_e4m3fn, device=dev)
-    la2 = torch.empty(M, R, dtype=torch.float32, device=dev)
-    svdq_gemm_w4a4(act=qx, wgt=t1["qweight"], out=out, qout=qout, ascales=asc, wscales=t1["wscales"], oscales=osc,
-                   lora_act_in=la, lora_up=t1["proj_up"], lora_down=t2["proj_down"], lora_act_out=la2, bias=t1["bias"],
-                   smooth_factor=t2["smooth_factor"], fp4=True, alpha=m1.alpha, wcscales=t1["wcscales"])
-    torch.cuda.synchronize()
+    la2 = torch.full((M, R), float("nan"), dtype=torch.float32, device=dev)
+
+    def run():
+        svdq_gemm_w4a4(act=qx, wgt=t1["qweight"], out=out, qout=qout, ascales=asc, wscales=t1["wscales"], oscales=osc,
+                       lora_act_in=la, lora_up=t1["proj_up"], lora_down=t2["proj_down"], lora_act_out=la2, bias=t1["bias"],
+                       smooth_factor=t2["smooth_factor"], fp4=True, alpha=m1.alpha, wcscales=t1["wcscales"])
+        torch.cuda.synchronize()
+
+    run()
+    first = la2.clone()
+    for _ in range(2):
+        la2.fill_(float("nan"))
+        run()
+        assert torch.equal(la2, first), "the next layer's low-rank input changed between two launches"
     h = out.cpu()
     want_codes, want_scales = quant.quantize_act_nvfp4(h, fc2.smooth)
     assert torch.equal(packing.act_to_logical(qout.cpu(), N1, fp4=True).to(torch.uint8), want_codes)
