@@ -120,7 +120,7 @@ struct GemmParams {
     void *oscales;               // bf16 [N/64, M_pad] or fp8 [N/16, M_pad]
     const float *next_smooth_rcp;  // fp32 [N]
     const bf16x8_t *next_down;   // native proj_down of the next layer ([N, R_down])
-    float *next_lora_out;        // fp32 [M_pad, R_down], zeroed before the launch, accumulated atomically
+    float *next_lora_out;        // fp32 [M_pad, R_down], written by the kernel that adds the shares behind the GEMM
     // tiles shared by two workgroups: parked partial sums (fp32 [2 * workgroups][256 threads][64] x 4)
     // and one arrival counter per tile (zero between launches)
     float *partials;
