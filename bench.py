@@ -82,11 +82,13 @@ def main():
     ap.add_argument("--qkv-rope", action="store_true",
                     help="time the GEMM with the RMS-norm + rotary epilogue of fused_qkv_norm_rottary (workload flux_qkv); "
                          "the CPU comparison is skipped")
-    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "awq-gemv", "fused-mlp"], default=None,
+    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "awq-gemv", "fused-mlp", "litela"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
                          "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters; "
                          "'awq-gemv' times the AWQ W4A16 GEMV at the modulation shape (1 row, K=3072, N=18432); "
-                         "'fused-mlp' times fused_gelu_mlp on the FLUX MLP pair (M=4608, 3072 -> 12288 -> 3072)")
+                         "'fused-mlp' times fused_gelu_mlp on the FLUX MLP pair (M=4608, 3072 -> 12288 -> 3072); "
+                         "'litela' times the linear-attention pair (QKV projection with the q / vk epilogue, then vk times q) at "
+                         "4096 tokens, K=2304, 72 heads of 32")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -118,6 +120,35 @@ def main():
         torch.cuda.synchronize()
         print(f"fused-mlp M={M} {K}->{N}->{K} rank {R}: {e0.elapsed_time(e1) * 1e3 / args.steps:.1f} us per call "
               "(quantize + fc1 with GELU / next-layer quantize / low-rank-down epilogue + fc2)")
+        return
+    if args.only == "litela":
+        from nunchaku_amd.models.linear import SVDQW4A4Linear
+        from nunchaku_amd.ops import linearattn_vk_mul_q, svdq_gemm_w4a4
+        from oracle import synth
+
+        dev = torch.device("cuda:0")
+        T, K, heads, R = 4096, 2304, 72, 32
+        N = heads * 96
+        mod = SVDQW4A4Linear(K, N, rank=R, device=dev)
+        mod.load_state_dict(synth.to_reference_checkpoint(synth.make_layer(N, K, R, seed=1)))
+        t = mod.native_tensors()
+        qx, asc, la = mod.quantize(synth.make_activations(T, K, seed=1).to(dev))
+        out = torch.empty(T, N, dtype=torch.bfloat16, device=dev)
+        q = torch.empty(1, T, N // 3, dtype=torch.bfloat16, device=dev)
+        vk = torch.empty(1, heads, 33, 32, dtype=torch.float32, device=dev)
+        base = dict(act=qx, wgt=t["qweight"], ascales=asc, wscales=t["wscales"], lora_act_in=la, lora_up=t["proj_up"], bias=t["bias"])
+        for name, fn in (("plain layer of the shape", lambda: svdq_gemm_w4a4(**base, out=out)),
+                         ("projection with relu(q) and vk sums", lambda: svdq_gemm_w4a4(**base, out_vk=vk, out_linearattn=q)),
+                         ("vk times q", lambda: linearattn_vk_mul_q(q, vk))):
+            for _ in range(20):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            print(f"litela T={T} K={K} heads={heads} rank {R}: {name}: {e0.elapsed_time(e1) * 1e3 / args.steps:.1f} us per call")
         return
     if args.only == "awq-gemv":
         from nunchaku_amd.ops import awq_gemv_w4a16

@@ -205,7 +205,7 @@ typedef struct svdq_gemm_args {
      *   out_vk[b][head][32][j] = sum of relu(k[row][j]),
      * on the bf16-rounded values, accumulated in fp32.  Every row of the GEMM counts, padding rows included, as in
      * the reference.  out_vk is fully written (the reference clears it first and adds with atomics in the order of
-     * arrival, :335, :649): every 32-row slab leaves its sums in the workspace and a small kernel launched behind the
+     * arrival, :335, :649): every row block of a workgroup leaves its sums in the workspace and a small kernel launched behind the
      * GEMM adds them in ascending order, so the result is the same from run to run.                             */
     float *out_vk;          /* fp32 [M_pad / vk_rows][2 N / 3 / 64][33][32]                                   */
     int64_t vk_rows;        /* rows per batch entry: a multiple of 256 that divides M_pad                     */

@@ -67,7 +67,7 @@ __global__ void __launch_bounds__(256) reduce_shares_kernel(const float4_t *part
     for (int e = 0; e < 4; e++) out[(size_t)(row + e) * R + rank] = sum[e];
 }
 
-// Sums the linear-attention shares of the 32-row slabs of a GEMM launch (gemm6_kernel.h; per slab and head 1056 floats:
+// Sums the linear-attention shares of the row blocks of a GEMM launch (gemm_params.h; per row block and head 1056 floats:
 // the 32 x 32 part [i][j] in the order of the matrix instruction's result registers, element e of lane l at
 // ((e / 4) * 64 + l) * 4 + e % 4 with i = 8 (e / 4) + 4 (l / 32) + e % 4, j = l % 32; then the 32 column sums) into
 // out_vk [batch][head][33][32].
@@ -270,7 +270,7 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     const size_t cnt_bytes = (size_t)ntiles * 4;
     const size_t part_bytes = kparts > 1 ? (size_t)ntiles * kparts * g6::BM * g6::BN * 4 : 0;
     const size_t share_bytes = p.next_down ? (size_t)nblocks * p.M_pad * p.R_down * 4 : 0;  // every column block's share of the next projection
-    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * VK_HEAD_FLOATS * 4 : 0;  // every 32-row slab's linear-attention sums
+    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / g6::BM) * (p.N / 96) * VK_HEAD_FLOATS * 4 : 0;  // every row block's linear-attention sums
     if (kparts == 1 && !p.next_down && !p.vk) return next ? g6::launch_next(p, ntiles, st) : g6::launch_plain(p, ntiles, st);
     std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
     if (!noalloc) lock.lock();
@@ -291,10 +291,10 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
         rc = check_launch("gemm_w4a4 (low-rank shares)");
     }
     if (rc == SVDQ_OK && p.vk) {
-        // the slabs' linear-attention sums, added per batch entry in ascending order of the rows
+        // the row blocks' linear-attention sums, added per batch entry in ascending order of the rows
         const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * VK_HEAD_FLOATS;
         hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
-                           p.vk_rows / 32, heads);
+                           p.vk_rows / g6::BM, heads);
         rc = check_launch("gemm_w4a4 (linear-attention sums)");
     }
     if (rc != SVDQ_OK && w.owner) w.owner->dirty = true;
@@ -361,9 +361,9 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     p.next_lora_part = nullptr;
     const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu || a->out_vk != nullptr;
     const bool shared_tiles = !(nwg <= ntiles && ntiles % nwg == 0);
-    // every 128-column chunk's share of the next layer's low-rank projection, every 32-row slab's linear-attention sums
+    // every 128-column chunk's share of the next layer's low-rank projection, every row block's linear-attention sums
     const size_t share_bytes = p.next_down ? (size_t)(p.N / 128) * p.M_pad * p.R_down * 4 : 0;
-    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * VK_HEAD_FLOATS * 4 : 0;
+    const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * VK_HEAD_FLOATS * 4 : 0;  // (this kernel: per 32-row slab)
     if (!shared_tiles && !share_bytes && !vk_bytes) return next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
     std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
     if (!noalloc) lock.lock();

@@ -432,6 +432,8 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     const bool interior = m0 + BM <= p.M_out && n0 + BN <= p.N_out;  // the whole tile lies inside the output
     uint16_t *slab = (uint16_t *)(lds + wave * SLAB_BYTES);
     const int ngroups_out = p.N / 64;
+    VkSums vks;  // linear attention: the sums of the wave's two slabs
+    if (NEXT && p.vk) litela_clear(vks);
     // one 32-row slab of the wave tile, instantiated twice with a compile-time slab index
     auto slab_epilogue = [&](auto MT) {
         constexpr int mt = decltype(MT)::value;
@@ -524,7 +526,7 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         __builtin_amdgcn_wave_barrier();
         // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores.  Streaming stores: the
         // tile is not read again by this kernel.
-        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) litela_slab(p.vk_part, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N);
+        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) litela_add_slab(vks, slab, OUT_LD, lane);
         if (NEXT && p.qkv.q && wcol0 < p.N) store_qkv_slab(p.qkv, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N / 3);
         if (p.out && interior) {  // no bounds to check: all slab reads first, then all stores
             u32x4_t d[8];
@@ -646,6 +648,12 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     __builtin_amdgcn_sched_barrier(0);
     slab_epilogue(std::integral_constant<int, 0>{});
     slab_epilogue(std::integral_constant<int, 1>{});
+    if (NEXT && p.vk && n0 + BN > p.N / 3) {
+        static_assert(SLAB_BYTES >= 2 * VK_HEAD_FLOATS * 4, "a wave's two heads pass through its slab area");
+        const int third = p.N / 3;
+        litela_finish(vks, wcol0 >= third && wcol0 < p.N, wm, wn, lds, SLAB_BYTES,
+                      p.vk_part + ((size_t)mb * (2 * third / 64) + (wcol0 - third) / 64) * VK_HEAD_FLOATS, lane);
+    }
 }
 
 template <bool NEXT>

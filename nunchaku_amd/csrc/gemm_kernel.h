@@ -731,7 +731,14 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         __builtin_amdgcn_wave_barrier();
         // EpilogueDefault (gemm_base.cuh:667-698): 16-byte row-contiguous stores.  Streaming stores: the
         // tile is not read again by this kernel.
-        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) litela_slab(p.vk_part, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N);
+        if (NEXT && p.vk && wcol0 >= p.N / 3 && wcol0 < p.N) {
+            // every 32-row slab parks its own sums (this kernel has no registers to carry them from slab to slab)
+            VkSums vks;
+            litela_clear(vks);
+            litela_add_slab(vks, slab, OUT_LD, lane);
+            const int third = p.N / 3;
+            litela_park<true>(vks, p.vk_part + ((size_t)((wrow0 + mt * 32) >> 5) * (2 * third / 64) + (wcol0 - third) / 64) * VK_HEAD_FLOATS, lane);
+        }
         if (NEXT && p.qkv.q && wcol0 < p.N) store_qkv_slab(p.qkv, slab, OUT_LD, lane, wrow0 + mt * 32, wcol0, p.N / 3);
         if (p.out && interior) {  // no bounds to check: all slab reads first, then all stores
             u32x4_t d[8];

@@ -58,24 +58,33 @@ __device__ inline void store_qkv_slab(const QkvOut &o, const uint16_t *slab, int
     }
 }
 
-// Linear attention (EpilogueLiteLA::apply_litela, epilogues.cuh:572-655) on one 32-row x 128-column bf16 slab in LDS
-// (rows `ld` elements apart): the 128 columns are two heads of [k 32 | v 32].  vk[i][j] = sum over the 32 rows of
-// v[row][i] * relu(k[row][j]) on the matrix cores (the rows are the contraction index: both operands are read down
-// the columns of the slab), row 32 = sum of relu(k[row][j]).  The slab's sums go to its own slot of the workspace
-// ([32-row slab][head] x 1056 floats, the 32 x 32 part in the lanes' order: a wave's store is 1 KB contiguous); a
-// small kernel behind the GEMM adds the slabs of a batch entry in ascending order (reduce_vk_kernel in gemm.hip).
+// Linear attention (EpilogueLiteLA::apply_litela, epilogues.cuh:572-655).  A wave's 128 output columns are two heads
+// of [k 32 | v 32].  vk[i][j] = sum over rows of v[row][i] * relu(k[row][j]) on the matrix cores (the rows are the
+// contraction index: both operands are read down the columns of the 32-row bf16 slab in LDS, rows `ld` elements
+// apart), row 32 = sum of relu(k[row][j]).  In the INT4 kernel a wave keeps the sums of its slabs in registers
+// (VkSums), the two waves of a column half meet in LDS, and the workgroup's row block goes to its own slot of the
+// workspace ([row block][head] x 1056 floats, the 32 x 32 part in the lanes' order: a wave's store is 1 KB contiguous);
+// the NVFP4 kernel parks every 32-row slab.  A small kernel behind the GEMM adds the row blocks of a batch entry in
+// ascending order (reduce_vk_kernel in gemm.hip).
 // The reference adds with atomics in the order of arrival (epilogues.cuh:649); atomics here, 2.4 M of them at 4096
 // rows and 72 heads, doubled the kernel's time.
 constexpr int VK_HEAD_FLOATS = 33 * 32;
-__device__ inline void litela_slab(float *vk_part, const uint16_t *slab, int ld, int lane, int row0, int col0, int N) {
-    const int j = lane & 31, kb = lane >> 5;
-    const int vheads = N / 3 * 2 / 64;
+struct VkSums {
+    float16_t d[2];  // per head: vk[i][j], element e of lane l is i = 8 (e / 4) + 4 (l / 32) + e % 4, j = l % 32
+    float ks[2];     // per head: this lane's part of the column sum of relu(k) for j = l % 32
+};
+__device__ inline void litela_clear(VkSums &s) {
 #pragma unroll
     for (int hd = 0; hd < 2; hd++) {
-        float16_t d;
 #pragma unroll
-        for (int e = 0; e < 16; e++) d[e] = 0.f;
-        float ks = 0.f;
+        for (int e = 0; e < 16; e++) s.d[hd][e] = 0.f;
+        s.ks[hd] = 0.f;
+    }
+}
+__device__ inline void litela_add_slab(VkSums &s, const uint16_t *slab, int ld, int lane) {
+    const int j = lane & 31, kb = lane >> 5;
+#pragma unroll
+    for (int hd = 0; hd < 2; hd++) {
 #pragma unroll
         for (int st = 0; st < 2; st++) {
             u32x4_t kw, vw;
@@ -88,19 +97,57 @@ __device__ inline void litela_slab(float *vk_part, const uint16_t *slab, int ld,
                     kk[f] = rowp[0];
                     vv[f] = rowp[32];
                     if (kk[f] & 0x8000u) kk[f] = 0;  // ReLU on the bf16 value
-                    ks += bits_f32(kk[f] << 16);
+                    s.ks[hd] += bits_f32(kk[f] << 16);
                 }
                 kw[e / 2] = kk[0] | (kk[1] << 16);
                 vw[e / 2] = vv[0] | (vv[1] << 16);
             }
-            d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vw), __builtin_bit_cast(bf16x8_t, kw), d, 0, 0, 0);
+            s.d[hd] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vw), __builtin_bit_cast(bf16x8_t, kw), s.d[hd], 0, 0, 0);
         }
-        ks += __shfl_xor(ks, 32);
-        float *dst = vk_part + ((size_t)(row0 >> 5) * vheads + (col0 - N / 3) / 64 + hd) * VK_HEAD_FLOATS;
+    }
+}
+// Writes the wave's two heads to dst (2 x 1056 floats, LDS or the workspace).
+template <bool STREAM>
+__device__ inline void litela_park(const VkSums &s, float *dst, int lane) {
+    const int j = lane & 31, kb = lane >> 5;
 #pragma unroll
-        for (int g = 0; g < 4; g++)
-            __builtin_nontemporal_store(float4_t{d[4 * g], d[4 * g + 1], d[4 * g + 2], d[4 * g + 3]}, (float4_t *)(dst + (g * 64 + lane) * 4));
-        if (kb == 0) dst[1024 + j] = ks;
+    for (int hd = 0; hd < 2; hd++) {
+        const float ks = s.ks[hd] + __shfl_xor(s.ks[hd], 32);
+        float *d = dst + hd * VK_HEAD_FLOATS;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4_t v = float4_t{s.d[hd][4 * g], s.d[hd][4 * g + 1], s.d[hd][4 * g + 2], s.d[hd][4 * g + 3]};
+            if (STREAM) __builtin_nontemporal_store(v, (float4_t *)(d + (g * 64 + lane) * 4));
+            else *(float4_t *)(d + (g * 64 + lane) * 4) = v;
+        }
+        if (kb == 0) d[1024 + j] = ks;
+    }
+}
+// s = s + what another wave parked at src (the rows of s come first).
+__device__ inline void litela_add_parked(VkSums &s, const float *src, int lane) {
+    const int j = lane & 31, kb = lane >> 5;
+#pragma unroll
+    for (int hd = 0; hd < 2; hd++) {
+        const float ks = s.ks[hd] + __shfl_xor(s.ks[hd], 32);
+        const float *d = src + hd * VK_HEAD_FLOATS;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4_t v = *(const float4_t *)(d + (g * 64 + lane) * 4);
+#pragma unroll
+            for (int i = 0; i < 4; i++) s.d[hd][4 * g + i] += v[i];
+        }
+        s.ks[hd] = kb == 0 ? ks + d[1024 + j] : 0.f;
+    }
+}
+// After the last slab of a tile, called by all four waves (2 x 2, wave = 2 wm + wn) when the tile holds k | v columns
+// (a condition uniform over the workgroup): the lower waves hand their sums to the upper ones through their own slab
+// areas, which they no longer need, and the upper ones store the row block's share.  `kv`: this wave's columns are k | v.
+__device__ inline void litela_finish(VkSums &s, bool kv, int wm, int wn, unsigned char *slabs, int slab_bytes, float *share, int lane) {
+    if (kv && wm == 1) litela_park<false>(s, (float *)(slabs + (2 + wn) * slab_bytes), lane);
+    __syncthreads();
+    if (kv && wm == 0) {
+        litela_add_parked(s, (const float *)(slabs + (2 + wn) * slab_bytes), lane);
+        litela_park<true>(s, share, lane);
     }
 }
 
@@ -201,7 +248,7 @@ struct Params {
     // stored through `out` after a ReLU; the rest is [head][k 32 | v 32]; vk[batch][head][i][j] += sum over the
     // tile's rows of v[i] relu(k[j]) (i < 32) and of relu(k[j]) (i = 32)
     float *vk;           // fp32 [batch][2 N / 3 / 64][33][32]; null: no such epilogue
-    float *vk_part;      // workspace: [M_pad / 32 slabs][heads] x 1056 floats, every slab's sums
+    float *vk_part;      // workspace: [M_pad / 128 row blocks][heads] x 1056 floats, every row block's sums
     int vk_rows;         // rows per batch entry, a multiple of 256
 };
 }  // namespace g6
