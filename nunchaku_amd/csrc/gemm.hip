@@ -71,28 +71,36 @@ __global__ void __launch_bounds__(256) reduce_shares_kernel(const float4_t *part
 // the 32 x 32 part [i][j] in the order of the matrix instruction's result registers, element e of lane l at
 // ((e / 4) * 64 + l) * 4 + e % 4 with i = 8 (e / 4) + 4 (l / 32) + e % 4, j = l % 32; then the 32 column sums) into
 // out_vk [batch][head][33][32].
-__global__ void __launch_bounds__(256) reduce_vk_kernel(const float *part, float *out, int batch, int slabs_per_batch, int heads) {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= batch * heads * VK_HEAD_FLOATS) return;
-    const int pos = idx % VK_HEAD_FLOATS, head = (idx / VK_HEAD_FLOATS) % heads, b = idx / (VK_HEAD_FLOATS * heads);
-    int src = pos;  // row 32: stored as it is
-    if (pos < 1024) {
-        const int i = pos >> 5, j = pos & 31;
-        const int g = i >> 3, kb = (i >> 2) & 1, e3 = i & 3;
-        src = (g * 64 + kb * 32 + j) * 4 + e3;
-    }
-    const float *p0 = part + ((size_t)b * slabs_per_batch * heads + head) * VK_HEAD_FLOATS + src;
-    const size_t stride = (size_t)heads * VK_HEAD_FLOATS;
+__global__ void __launch_bounds__(256) reduce_vk_kernel(const float *part, float *out, int batch, int blocks_per_batch, int heads) {
+    // 64 outputs per workgroup; the row blocks of an output are split over four threads (more requests in flight),
+    // whose sums are added in ascending order
+    __shared__ float quarter[4][64];
+    const int idx = blockIdx.x * 64 + (threadIdx.x & 63), qt = threadIdx.x >> 6;
+    const bool live = idx < batch * heads * VK_HEAD_FLOATS;
     float sum = 0.f;
-    for (int s0 = 0; s0 < slabs_per_batch; s0 += 8) {  // eight requests in flight
-        float v[8];
+    if (live) {
+        const int pos = idx % VK_HEAD_FLOATS, head = (idx / VK_HEAD_FLOATS) % heads, b = idx / (VK_HEAD_FLOATS * heads);
+        int src = pos;  // row 32: stored as it is
+        if (pos < 1024) {
+            const int i = pos >> 5, j = pos & 31;
+            const int g = i >> 3, kb = (i >> 2) & 1, e3 = i & 3;
+            src = (g * 64 + kb * 32 + j) * 4 + e3;
+        }
+        const float *p0 = part + ((size_t)b * blocks_per_batch * heads + head) * VK_HEAD_FLOATS + src;
+        const size_t stride = (size_t)heads * VK_HEAD_FLOATS;
+        const int per = (blocks_per_batch + 3) / 4, first = qt * per, last = first + per < blocks_per_batch ? first + per : blocks_per_batch;
+        for (int s0 = first; s0 < last; s0 += 8) {  // eight requests in flight
+            float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = p0[(size_t)(s0 + u < slabs_per_batch ? s0 + u : slabs_per_batch - 1) * stride];
+            for (int u = 0; u < 8; u++) v[u] = p0[(size_t)(s0 + u < last ? s0 + u : last - 1) * stride];
 #pragma unroll
-        for (int u = 0; u < 8; u++)
-            if (s0 + u < slabs_per_batch) sum += v[u];
+            for (int u = 0; u < 8; u++)
+                if (s0 + u < last) sum += v[u];
+        }
     }
-    out[idx] = sum;
+    quarter[qt][threadIdx.x & 63] = sum;
+    __syncthreads();
+    if (live && qt == 0) out[idx] = ((quarter[0][threadIdx.x] + quarter[1][threadIdx.x]) + quarter[2][threadIdx.x]) + quarter[3][threadIdx.x];
 }
 
 void clear_zero_region(Workspace *w) {
@@ -293,7 +301,7 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     if (rc == SVDQ_OK && p.vk) {
         // the row blocks' linear-attention sums, added per batch entry in ascending order of the rows
         const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * VK_HEAD_FLOATS;
-        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
+        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
                            p.vk_rows / g6::BM, heads);
         rc = check_launch("gemm_w4a4 (linear-attention sums)");
     }
@@ -386,7 +394,7 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     }
     if (rc == SVDQ_OK && p.vk) {
         const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * VK_HEAD_FLOATS;
-        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
+        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
                            p.vk_rows / 32, heads);
         rc = check_launch("gemm_w4a4 (linear-attention sums)");
     }
