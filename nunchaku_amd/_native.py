@@ -170,6 +170,19 @@ def stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+def launch(entry, args_ref, device: torch.device) -> None:
+    """Call ``entry(args, stream)`` of the C ABI on ``device``'s current stream.  The library launches on the
+    current device: the switch (and torch's stream object) is only paid for when ``device`` is not current."""
+    idx = device.index
+    if idx is not None and idx == torch.cuda.current_device():
+        rc = entry(args_ref, torch._C._cuda_getCurrentRawStream(idx))
+    else:
+        with torch.cuda.device(device):
+            rc = entry(args_ref, torch.cuda.current_stream(device).cuda_stream)
+    if rc:
+        check(rc)
+
+
 def ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 

@@ -8,12 +8,48 @@ tensors are what the kernels read.
 
 from __future__ import annotations
 
+import ctypes
+import threading
+
 import torch
 from torch import nn
 
+from .. import _native as nv
 from .. import packing
+from ..ops import gemm as _gemm_op
 from ..ops.gemm import svdq_gemm_w4a4
 from ..ops.quantize import svdq_quantize_w4a4_act_fuse_lora
+
+
+class _LayerCall:
+    """The argument blocks of a layer's two C-ABI calls with everything filled in that does not change from one
+    forward to the next (the layer's own tensors and sizes); ``SVDQW4A4Linear.forward`` only sets the pointers and
+    row counts of the call.  The layer's tensors were checked when they were converted; the per-call tensors are
+    allocated by ``forward`` itself, so the checks of the operator wrappers have nothing left to find."""
+
+    def __init__(self, mod: "SVDQW4A4Linear", t: dict):
+        fp4 = mod.precision == "nvfp4"
+        K, N, R = mod.in_features, mod.out_features, mod.rank
+        self.fp4 = fp4
+        self.act_bytes = packing.act_nbytes_per_row(K, fp4)
+        self.groups = K // mod.group_size
+        self.scale_dtype = torch.float8_e4m3fn if fp4 else torch.bfloat16
+        self.tensors = t  # keeps the converted tensors alive as long as their addresses are in the blocks
+        self.q = nv.QuantizeArgs(
+            lora_down=nv.ptr(t["proj_down"]) if R else None, smooth_rcp=nv.ptr(t["smooth_factor"]),
+            K=K, R=R, fp4=int(fp4), fuse_glu=0,
+        )
+        self.device = t["qweight"].device
+        self.sc = (ctypes.c_float * max(1, (R + 15) // 16))()
+        self.scales_src = ()  # what self.sc was last written from (never a list or None: the first call writes)
+        self.g = nv.GemmArgs(
+            wgt=nv.ptr(t["qweight"]), wscales=nv.ptr(t["wscales"]), colnorm=nv.ptr(t["wscales"].colnorm), bias=nv.ptr(t["bias"]),
+            wcscales=nv.ptr(t["wcscales"]), lora_up=nv.ptr(t["proj_up"]) if R else None, lora_scales=self.sc,
+            N=N, K=K, N_out=N, R_up=R, R_down=0, alpha=float(mod.alpha), act_unsigned=int(mod.act_unsigned), fuse_silu=0, fp4=int(fp4),
+            norm_eps=_gemm_op.NORM_EPS,
+        )
+        self.q_ref, self.g_ref = ctypes.byref(self.q), ctypes.byref(self.g)
+        self.lock = threading.Lock()  # the blocks are shared by the threads that call the layer
 
 
 class SVDQW4A4Linear(nn.Module):
@@ -71,6 +107,7 @@ class SVDQW4A4Linear(nn.Module):
         self._native: dict[str, torch.Tensor | None] | None = None
         self._native_stamp: tuple | None = None
         self._alpha: float | None = None
+        self._call: _LayerCall | None = None
 
     @classmethod
     def from_linear(cls, linear: nn.Linear, **kwargs):
@@ -97,9 +134,10 @@ class SVDQW4A4Linear(nn.Module):
 
     def _stamp(self) -> tuple:
         """Identity and in-place modification counter of every parameter the native tensors come from."""
+        params = self._parameters  # (nn.Module.__getattr__ is a slow way to the same dictionary)
         out = []
         for name in self._NATIVE_SOURCES:
-            t = getattr(self, name, None)
+            t = params.get(name)
             out.append(None if t is None else (t.data_ptr(), packing.tensor_version(t)))
         return tuple(out)
 
@@ -111,6 +149,7 @@ class SVDQW4A4Linear(nn.Module):
         self._native = None
         self._native_stamp = None
         self._alpha = None
+        self._call = None
 
     def native_tensors(self) -> dict[str, torch.Tensor | None]:
         """The layer's tensors in the layouts the kernels read, converted on first use and again after
@@ -156,6 +195,7 @@ class SVDQW4A4Linear(nn.Module):
             raise ValueError("skip_ranks must be a multiple of 16")
         groups = (self.rank + 15) // 16
         self.lora_scales = [1.0 if i < skip_ranks // 16 else float(scale) for i in range(groups)]
+        self._call = None
 
     @property
     def alpha(self) -> float:
@@ -168,13 +208,60 @@ class SVDQW4A4Linear(nn.Module):
 
     # ---- forward path (nunchaku/models/linear.py:89-132) ----------------------------------------
     def forward(self, x: torch.Tensor, output: torch.Tensor | None = None) -> torch.Tensor:
+        """``quantize`` then ``forward_quant`` (nunchaku/models/linear.py:89-110), through argument blocks prepared
+        once per layer: a forward costs the host four allocations and two calls into the library."""
         batch_size, seq_len, channels = x.shape
-        x = x.view(batch_size * seq_len, channels)
+        M = batch_size * seq_len
+        x = x.view(M, channels)
+        dev = x.device
+        if not x.is_cuda:
+            raise RuntimeError(f"x must live on a GPU (got {dev}); this path has no CPU implementation")
+        if not x.is_contiguous():
+            raise ValueError("x must be contiguous")
+        if M == 0:
+            return self._forward_by_operators(x, output).view(batch_size, seq_len, -1)
+        if x.dtype != torch.bfloat16:
+            raise NotImplementedError("only bf16 activations are supported")
+        if channels != self.in_features:
+            raise ValueError(f"x has {channels} channels, the layer takes {self.in_features}")
         if output is None:
-            output = torch.empty(batch_size * seq_len, self.out_features, dtype=x.dtype, device=x.device)
-        quantized_x, ascales, lora_act_out = self.quantize(x)
-        output = self.forward_quant(quantized_x, ascales, lora_act_out, output)
+            output = torch.empty(M, self.out_features, dtype=x.dtype, device=dev)
+        elif not (output.is_cuda and output.device == dev and output.dtype == torch.bfloat16 and output.is_contiguous()
+                  and output.numel() == M * self.out_features and output.shape[-1] == self.out_features):
+            raise ValueError(f"output must be a contiguous bf16 tensor of {M} x {self.out_features} elements on {dev}")
+        t = self.native_tensors()
+        c = self._call
+        if c is None:
+            c = self._call = _LayerCall(self, t)
+        if c.device != dev:
+            raise ValueError(f"x is on {dev}, the layer on {c.device}")
+        M_pad = (M + 255) // 256 * 256
+        qx = torch.empty(M_pad, c.act_bytes, dtype=torch.uint8, device=dev)
+        ascales = torch.empty(c.groups, M_pad, dtype=c.scale_dtype, device=dev)
+        lora_act = torch.empty(M_pad, self.rank, dtype=torch.float32, device=dev)
+        lib = nv.lib()
+        with c.lock:
+            q, g = c.q, c.g
+            ls = self.lora_scales
+            if ls is not None or c.scales_src is not None:  # one factor per 16 ranks; missing entries count as zero, None as all ones
+                for i in range(len(c.sc)):
+                    c.sc[i] = 1.0 if ls is None else (float(ls[i]) if i < len(ls) else 0.0)
+                c.scales_src = ls
+            q.input, q.output, q.oscales = x.data_ptr(), qx.data_ptr(), ascales.data_ptr()
+            q.lora_act_out = lora_act.data_ptr() if self.rank else None
+            q.M, q.M_pad = M, M_pad
+            g.act, g.ascales, g.out = q.output, q.oscales, output.data_ptr()
+            g.lora_act_in = q.lora_act_out
+            g.M_pad, g.M_out = M_pad, M
+            g.k_split = int(_gemm_op.K_SPLIT or 0)
+            nv.launch(lib.svdq_quantize_w4a4_act_fuse_lora, c.q_ref, dev)
+            nv.launch(lib.svdq_gemm_w4a4_noalloc if _gemm_op.NO_ALLOC else lib.svdq_gemm_w4a4, c.g_ref, dev)
         return output.view(batch_size, seq_len, -1)
+
+    def _forward_by_operators(self, x: torch.Tensor, output: torch.Tensor | None) -> torch.Tensor:
+        """The same through the two operator wrappers (every argument checked on every call)."""
+        quantized_x, ascales, lora_act_out = self.quantize(x)
+        return self.forward_quant(quantized_x, ascales, lora_act_out, output)
 
     def quantize(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         t = self.native_tensors()

@@ -230,9 +230,7 @@ def svdq_gemm_w4a4(
         attn_tokens=int(attn_tokens) if out_q is not None else 0, qkv_rows=M_pad if out_q is not None else 0,
         out_vk=nv.ptr(out_vk), vk_rows=vk_rows,
     )
-    with torch.cuda.device(dev):  # the library launches on the current device
-        entry = nv.lib().svdq_gemm_w4a4_noalloc if NO_ALLOC else nv.lib().svdq_gemm_w4a4
-        nv.check(entry(ctypes.byref(args), nv.stream_ptr(dev)))
+    nv.launch(nv.lib().svdq_gemm_w4a4_noalloc if NO_ALLOC else nv.lib().svdq_gemm_w4a4, ctypes.byref(args), dev)
 
 
 svdq_gemm_w4a4_cuda = svdq_gemm_w4a4

@@ -48,7 +48,7 @@ def awq_gemv_w4a16(
         x=in_feats.data_ptr(), qweight=kernel.data_ptr(), scales=scaling_factors.data_ptr(), zeros=zeros.data_ptr(),
         bias=nv.ptr(bias), out=out.data_ptr(), M=m, N=n, K=k, group_size=group_size,
     )
-    nv.check(nv.lib().svdq_awq_gemv_w4a16(ctypes.byref(args), nv.stream_ptr(in_feats.device)))
+    nv.launch(nv.lib().svdq_awq_gemv_w4a16, ctypes.byref(args), in_feats.device)
     return out
 
 

@@ -88,8 +88,7 @@ def svdq_quantize_w4a4_act_fuse_lora(
         lora_down=nv.ptr(down) if rank else None, lora_act_out=lora_act_out.data_ptr() if rank else None, smooth_rcp=nv.ptr(rcp),
         M=batch_size, M_pad=batch_size_pad, K=channels, R=rank, fp4=int(fp4), fuse_glu=int(fuse_glu),
     )
-    with torch.cuda.device(dev):  # the library launches on the current device
-        nv.check(nv.lib().svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(args), nv.stream_ptr(dev)))
+    nv.launch(nv.lib().svdq_quantize_w4a4_act_fuse_lora, ctypes.byref(args), dev)
     return output, oscales, lora_act_out
 
 

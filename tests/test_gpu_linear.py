@@ -137,3 +137,36 @@ def test_batched_rank128_shape_properties(dev):
     """M=18432 (4 x 4608 tokens), K=3072, N=12288, rank 128: several batches of tiles per workgroup and
     four rounds of the low-rank up projection."""
     _full_shape_properties(dev, "c5", sample_rows=128)
+
+
+@pytest.mark.parametrize("fp4", [False, True])
+def test_forward_equals_the_two_operators(dev, fp4):
+    """``forward`` goes through argument blocks prepared once per layer; the operator wrappers check and build
+    everything per call.  Same bits, for row counts that change from call to call, a caller's output buffer,
+    per-rank factors assigned as an attribute and a low-rank swap in between."""
+    announce(f"forward against quantize + forward_quant, fp4={fp4}")
+    layer = synth.make_layer(384, 256, 32, seed=31, fp4=fp4)
+    m = make_module(layer, dev)
+    for rows in (300, 75, 512):
+        x = synth.make_activations(rows, 256, seed=rows).to(dev)
+        want = m._forward_by_operators(x, None)
+        got = m(x.view(1, rows, 256))
+        assert torch.equal(got[0], want[:rows])  # (forward_quant without an output returns the padded rows)
+    buf = torch.full((2, 75, 384), 7.0, dtype=torch.bfloat16, device=dev)
+    x = synth.make_activations(150, 256, seed=5).to(dev)
+    assert m(x.view(2, 75, 256), buf).data_ptr() == buf.data_ptr()
+    assert torch.equal(buf.view(150, 384), m._forward_by_operators(x, None)[:150])
+    m.lora_scales = [1.0, 0.25]
+    assert torch.equal(m(x.view(1, 150, 256))[0], m._forward_by_operators(x, None)[:150])
+    m.lora_scales = None
+    from nunchaku_amd.checkpoint import concat_lowrank
+
+    m.update_lora(concat_lowrank(m.proj_down.data, m.proj_down.data), concat_lowrank(m.proj_up.data, -m.proj_up.data))  # rank 64
+    m.set_lora_scale(32, 0.5)
+    assert torch.equal(m(x.view(1, 150, 256))[0], m._forward_by_operators(x, None)[:150])
+    with pytest.raises(ValueError):
+        m(x.view(1, 150, 256)[:, :, :128])
+    with pytest.raises(ValueError):
+        m(x.view(1, 150, 256), torch.empty(150, 385, dtype=torch.bfloat16, device=dev))
+    with pytest.raises(RuntimeError):
+        m(x.cpu().view(1, 150, 256))
