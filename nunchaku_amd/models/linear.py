@@ -213,50 +213,79 @@ class SVDQW4A4Linear(nn.Module):
         batch_size, seq_len, channels = x.shape
         M = batch_size * seq_len
         x = x.view(M, channels)
-        dev = x.device
-        if not x.is_cuda:
-            raise RuntimeError(f"x must live on a GPU (got {dev}); this path has no CPU implementation")
-        if not x.is_contiguous():
-            raise ValueError("x must be contiguous")
         if M == 0:
             return self._forward_by_operators(x, output).view(batch_size, seq_len, -1)
-        if x.dtype != torch.bfloat16:
-            raise NotImplementedError("only bf16 activations are supported")
-        if channels != self.in_features:
-            raise ValueError(f"x has {channels} channels, the layer takes {self.in_features}")
+        c = self._prepared(x)
+        dev = c.device
         if output is None:
             output = torch.empty(M, self.out_features, dtype=x.dtype, device=dev)
         elif not (output.is_cuda and output.device == dev and output.dtype == torch.bfloat16 and output.is_contiguous()
                   and output.numel() == M * self.out_features and output.shape[-1] == self.out_features):
             raise ValueError(f"output must be a contiguous bf16 tensor of {M} x {self.out_features} elements on {dev}")
+        M_pad = (M + 255) // 256 * 256
+        qx, ascales, lora_act = self._quantize_prepared(c, x, M_pad)
+        self._gemm_prepared(c, qx, ascales, lora_act, M_pad, out=output.data_ptr(), M_out=M)
+        return output.view(batch_size, seq_len, -1)
+
+    # The three steps of ``forward``, also used by ``ops.fused``: no argument is checked twice, none is looked up twice.
+    def _prepared(self, x: torch.Tensor) -> _LayerCall:
+        """Checks the activations ``x`` [M, K] against the layer and returns the layer's argument blocks."""
+        if not x.is_cuda:
+            raise RuntimeError(f"x must live on a GPU (got {x.device}); this path has no CPU implementation")
+        if not x.is_contiguous():
+            raise ValueError("x must be contiguous")
+        if x.dtype != torch.bfloat16:
+            raise NotImplementedError("only bf16 activations are supported")
+        if x.shape[-1] != self.in_features:
+            raise ValueError(f"x has {x.shape[-1]} channels, the layer takes {self.in_features}")
+        return self._blocks(x.device)
+
+    def _blocks(self, dev: torch.device) -> _LayerCall:
         t = self.native_tensors()
         c = self._call
         if c is None:
             c = self._call = _LayerCall(self, t)
         if c.device != dev:
-            raise ValueError(f"x is on {dev}, the layer on {c.device}")
-        M_pad = (M + 255) // 256 * 256
+            raise ValueError(f"the activations are on {dev}, the layer on {c.device}")
+        return c
+
+    def _quantize_prepared(self, c: _LayerCall, x: torch.Tensor, M_pad: int):
+        dev = c.device
         qx = torch.empty(M_pad, c.act_bytes, dtype=torch.uint8, device=dev)
         ascales = torch.empty(c.groups, M_pad, dtype=c.scale_dtype, device=dev)
         lora_act = torch.empty(M_pad, self.rank, dtype=torch.float32, device=dev)
+        with c.lock:
+            q = c.q
+            q.input, q.output, q.oscales = x.data_ptr(), qx.data_ptr(), ascales.data_ptr()
+            q.lora_act_out = lora_act.data_ptr() if self.rank else None
+            q.M, q.M_pad = x.shape[0], M_pad
+            nv.launch(nv.lib().svdq_quantize_w4a4_act_fuse_lora, c.q_ref, dev)
+        return qx, ascales, lora_act
+
+    def _gemm_prepared(self, c: _LayerCall, qx: torch.Tensor, ascales: torch.Tensor, lora_act: torch.Tensor, M_pad: int,
+                       out: int | None = None, M_out: int = 0, **epilogue) -> None:
+        """The layer's GEMM on quantized activations made for it (``_quantize_prepared``, or another layer's
+        next-layer epilogue).  ``out``: address of a bf16 [M_out, N] buffer.  ``epilogue``: further fields of the
+        argument block (addresses and sizes), in force for this call only."""
         lib = nv.lib()
         with c.lock:
-            q, g = c.q, c.g
+            g = c.g
             ls = self.lora_scales
             if ls is not None or c.scales_src is not None:  # one factor per 16 ranks; missing entries count as zero, None as all ones
                 for i in range(len(c.sc)):
                     c.sc[i] = 1.0 if ls is None else (float(ls[i]) if i < len(ls) else 0.0)
                 c.scales_src = ls
-            q.input, q.output, q.oscales = x.data_ptr(), qx.data_ptr(), ascales.data_ptr()
-            q.lora_act_out = lora_act.data_ptr() if self.rank else None
-            q.M, q.M_pad = M, M_pad
-            g.act, g.ascales, g.out = q.output, q.oscales, output.data_ptr()
-            g.lora_act_in = q.lora_act_out
-            g.M_pad, g.M_out = M_pad, M
+            g.act, g.ascales, g.out = qx.data_ptr(), ascales.data_ptr(), out
+            g.lora_act_in = lora_act.data_ptr() if self.rank else None
+            g.M_pad, g.M_out = M_pad, M_out
             g.k_split = int(_gemm_op.K_SPLIT or 0)
-            nv.launch(lib.svdq_quantize_w4a4_act_fuse_lora, c.q_ref, dev)
-            nv.launch(lib.svdq_gemm_w4a4_noalloc if _gemm_op.NO_ALLOC else lib.svdq_gemm_w4a4, c.g_ref, dev)
-        return output.view(batch_size, seq_len, -1)
+            for name, value in epilogue.items():
+                setattr(g, name, value)
+            try:
+                nv.launch(lib.svdq_gemm_w4a4_noalloc if _gemm_op.NO_ALLOC else lib.svdq_gemm_w4a4, c.g_ref, c.device)
+            finally:
+                for name in epilogue:
+                    setattr(g, name, 0 if name in ("R_down",) else None)
 
     def _forward_by_operators(self, x: torch.Tensor, output: torch.Tensor | None) -> torch.Tensor:
         """The same through the two operator wrappers (every argument checked on every call)."""

@@ -4,35 +4,38 @@ from __future__ import annotations
 
 import torch
 
-from ..packing import act_nbytes_per_row
 from ..utils import ceil_divide
 from .gemm import svdq_gemm_w4a4
 
 
 def fused_gelu_mlp(x: torch.Tensor, fc1, fc2, pad_size: int = 256) -> torch.Tensor:
     """fc1 -> GELU -> fc2 with the GELU, fc2's activation quantization (unsigned INT4 after a
-    +0.171875 shift) and fc2's low-rank down projection fused into fc1's GEMM epilogue."""
+    +0.171875 shift) and fc2's low-rank down projection fused into fc1's GEMM epilogue
+    (nunchaku/ops/fused.py:10-47).  Three calls into the library through the layers' prepared argument blocks."""
     batch_size, seq_len, channels = x.shape
-    x = x.view(batch_size * seq_len, channels)
-    quantized_x, ascales, lora_act = fc1.quantize(x)
-
-    batch_size_pad = ceil_divide(batch_size * seq_len, pad_size) * pad_size
-    qout_act = torch.empty(batch_size_pad, act_nbytes_per_row(fc1.out_features, fc2.precision == "nvfp4"), dtype=torch.uint8, device=x.device)
-    if fc2.precision == "nvfp4":
-        qout_ascales = torch.empty(fc1.out_features // 16, batch_size_pad, dtype=torch.float8_e4m3fn, device=x.device)
-    else:
-        qout_ascales = torch.empty(fc1.out_features // 64, batch_size_pad, dtype=x.dtype, device=x.device)
-    qout_lora_act = torch.empty(batch_size_pad, fc2.proj_down.shape[1], dtype=torch.float32, device=x.device)
-
-    t1, t2 = fc1.native_tensors(), fc2.native_tensors()
-    svdq_gemm_w4a4(
-        act=quantized_x, wgt=t1["qweight"], qout=qout_act, ascales=ascales, wscales=t1["wscales"],
-        oscales=qout_ascales, lora_act_in=lora_act, lora_up=t1["proj_up"], lora_down=t2["proj_down"],
-        lora_act_out=qout_lora_act, bias=t1["bias"], smooth_factor=t2["smooth_factor"],
-        fp4=fc1.precision == "nvfp4", alpha=fc1.alpha, wcscales=t1["wcscales"], lora_scales=fc1.lora_scales,
+    M = batch_size * seq_len
+    x = x.view(M, channels)
+    if pad_size % 256 != 0:
+        raise ValueError("pad_size must be a multiple of 256")
+    if fc1.out_features != fc2.in_features or fc1.precision != fc2.precision:
+        raise ValueError(f"fc2 ({fc2}) does not take what fc1 ({fc1}) gives")
+    if M == 0:
+        return x.new_empty(batch_size, seq_len, fc2.out_features)
+    c1 = fc1._prepared(x)
+    dev = c1.device
+    c2 = fc2._blocks(dev)
+    M_pad = ceil_divide(M, pad_size) * pad_size
+    quantized_x, ascales, lora_act = fc1._quantize_prepared(c1, x, M_pad)
+    qout_act = torch.empty(M_pad, c2.act_bytes, dtype=torch.uint8, device=dev)
+    qout_ascales = torch.empty(c2.groups, M_pad, dtype=c2.scale_dtype, device=dev)
+    qout_lora_act = torch.empty(M_pad, fc2.rank, dtype=torch.float32, device=dev)
+    fc1._gemm_prepared(
+        c1, quantized_x, ascales, lora_act, M_pad,
+        qout=qout_act.data_ptr(), oscales=qout_ascales.data_ptr(), next_smooth_rcp=c2.q.smooth_rcp,
+        next_lora_down=c2.q.lora_down, next_lora_act_out=qout_lora_act.data_ptr() if fc2.rank else None, R_down=fc2.rank,
     )
-    output = torch.empty(batch_size * seq_len, fc2.out_features, dtype=x.dtype, device=x.device)
-    output = fc2.forward_quant(qout_act, qout_ascales, qout_lora_act, output=output)
+    output = torch.empty(M, fc2.out_features, dtype=x.dtype, device=dev)
+    fc2._gemm_prepared(c2, qout_act, qout_ascales, qout_lora_act, M_pad, out=output.data_ptr(), M_out=M)
     return output.view(batch_size, seq_len, -1)
 
 
@@ -46,11 +49,12 @@ def fused_qkv_norm_rottary(x: torch.Tensor, proj, norm_q, norm_k, rotary_emb: to
     masked (see ``svdq_gemm_w4a4``)."""
     batch_size, seq_len, channels = x.shape
     x = x.view(batch_size * seq_len, channels)
-    quantized_x, ascales, lora_act = proj.quantize(x)
-    t = proj.native_tensors()
+    c = proj._prepared(x)
+    quantized_x, ascales, lora_act = proj._quantize_prepared(c, x, ceil_divide(x.shape[0], 256) * 256)
+    t = c.tensors
     common = dict(
         act=quantized_x, wgt=t["qweight"], ascales=ascales, wscales=t["wscales"], lora_act_in=lora_act, lora_up=t["proj_up"],
-        bias=t["bias"], fp4=proj.precision == "nvfp4", alpha=proj.alpha, wcscales=t["wcscales"], norm_q=norm_q.weight,
+        bias=t["bias"], fp4=c.fp4, alpha=c.g.alpha, wcscales=t["wcscales"], norm_q=norm_q.weight,
         norm_k=norm_k.weight, rotary_emb=rotary_emb, lora_scales=proj.lora_scales,
     )
     if isinstance(output, tuple):
