@@ -30,6 +30,18 @@ class _LayerCall:
     def __init__(self, mod: "SVDQW4A4Linear", t: dict):
         fp4 = mod.precision == "nvfp4"
         K, N, R = mod.in_features, mod.out_features, mod.rank
+        # the kernels read every element these sizes promise: parameters assigned by hand must keep them
+        # (load_state_dict and update_lora check on their own)
+        sdt = torch.float8_e4m3fn if fp4 else torch.bfloat16
+        for name, shape, dtype in (("qweight", (N, K // 2), torch.int8), ("wscales", (K // mod.group_size, N), sdt),
+                                   ("smooth_factor", (K,), torch.bfloat16), ("proj_down", (K, R), torch.bfloat16),
+                                   ("proj_up", (N, R), torch.bfloat16), ("bias", (N,), torch.bfloat16), ("wcscales", (N,), torch.bfloat16)):
+            p = mod._parameters.get(name)
+            if p is None and name in ("bias", "wcscales"):
+                continue
+            if p is None or tuple(p.shape) != shape or p.dtype != dtype:
+                raise ValueError(f"{name} must be {dtype} {shape} for in_features={K}, out_features={N}, rank={R}, got "
+                                 f"{None if p is None else (p.dtype, tuple(p.shape))}")
         self.fp4 = fp4
         self.act_bytes = packing.act_nbytes_per_row(K, fp4)
         self.groups = K // mod.group_size

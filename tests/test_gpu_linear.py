@@ -170,3 +170,14 @@ def test_forward_equals_the_two_operators(dev, fp4):
         m(x.view(1, 150, 256), torch.empty(150, 385, dtype=torch.bfloat16, device=dev))
     with pytest.raises(RuntimeError):
         m(x.cpu().view(1, 150, 256))
+
+
+def test_forward_refuses_a_parameter_of_the_wrong_shape(dev):
+    announce("forward with a hand-assigned parameter of the wrong shape")
+    layer = synth.make_layer(256, 256, 32, seed=33)
+    m = make_module(layer, dev)
+    x = synth.make_activations(256, 256, seed=33).to(dev).view(1, 256, 256)
+    m(x)
+    m.proj_up = torch.nn.Parameter(m.proj_up.data[:128].clone(), requires_grad=False)
+    with pytest.raises(ValueError):
+        m(x)
