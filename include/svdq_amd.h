@@ -216,8 +216,8 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
 /* The same operator for callers that cannot allocate device memory: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  It runs the
  * same kernels as svdq_gemm_w4a4 and gives the same results bit for bit, but calls that need a workspace
- * (see above) take it from a fixed array in device memory (42 MB on every GPU the library runs on, held
- * until the process ends: 10 MB for arrival counters, 32 MB for partial sums and low-rank shares) instead
+ * (see above) take it from a fixed array in device memory (81 MB on every GPU the library runs on, held
+ * until the process ends: 1 MB for arrival counters, 80 MB for partial sums and low-rank shares) instead
  * of allocating one: no hipMalloc, hipFree or other allocating call is made.  A call whose need exceeds
  * the array returns SVDQ_EUNSUPPORTED with a message that says how much it wanted (examples that fit:
  * INT4 M_pad = 256, K = N = 3072 split six ways (k_split = 6), 18.9 MB of partial sums; next_lora_down at

@@ -152,7 +152,7 @@ Workspace *get_workspace(int dev, hipStream_t stream, size_t zero_bytes, size_t 
 // ---- the scratch of svdq_gemm_w4a4_noalloc --------------------------------------------------------
 // A fixed array in device memory, one copy per GPU, held until the process ends: first the region that
 // must be zero when a launch starts (arrival counters), then parked partial sums and low-rank shares.
-constexpr size_t NOALLOC_ZERO_BYTES = 10u << 20, NOALLOC_SCRATCH_BYTES = 32u << 20;
+constexpr size_t NOALLOC_ZERO_BYTES = 1u << 20, NOALLOC_SCRATCH_BYTES = 80u << 20;
 static __device__ __align__(256) unsigned char scratch[NOALLOC_ZERO_BYTES + NOALLOC_SCRATCH_BYTES];
 uint8_t *g_scratch_ptr[64] = {nullptr};  // the array's device address on each GPU, asked once per GPU
 std::mutex g_scratch_mutex;
@@ -220,6 +220,31 @@ int compute_units(int dev) {
     return cached[dev];
 }
 
+// Into how many parts along K the tiles of an INT4 launch are split when the caller leaves that to the library.
+// Launches with more tiles than compute units are not split: every part parks 128 KB of sums and the last one fetches
+// them all, which only pays while compute units would otherwise stand idle.  Below that, a model of the time in us,
+// fitted to launches of 24 ... 216 tiles at K = 3072 and 12288 on 256 compute units: a k-group takes a workgroup 0.55 us
+// while it has its compute unit to itself and 0.95 us when two share one; prologue and epilogue 4.4; a split costs
+// 5.3 + 2.6 per part beyond the first, half as much again when compute units are shared.  Measured, whole / best
+// split: 24 tiles at K = 3072 30.8 / 23.8 (3 parts), 72 tiles 31.0 / 26.9 (3), 96 tiles 31.4 / 28.6 (2), 144 tiles
+// 31.8 / 36.7 (not split); K = 12288: 24 tiles 104.5 / 39.3 (6), 72 tiles 104.8 / 51.4 (3), 144 tiles 105.0 / 75.2 (3).
+int choose_kparts(int ntiles, int kgroups, int ncu) {
+    if (ntiles > ncu) return 1;
+    int best = 1;
+    double best_t = 0.55 * kgroups + 4.4;
+    for (int k : {2, 3, 4, 6, 8}) {
+        const int units = ntiles * k, g = (kgroups + k - 1) / k;
+        if (g < 12 || units > 2 * ncu) break;
+        const bool shared = units > ncu;
+        const double t = g * (shared ? 0.95 : 0.55) + 4.4 + (5.3 + 2.6 * (k - 1)) * (shared ? 1.5 : 1.0);
+        if (t < (best == 1 ? 0.90 : 0.95) * best_t) {  // a split has to pay clearly; more parts likewise
+            best = k;
+            best_t = t;
+        }
+    }
+    return best;
+}
+
 // ---- INT4: fp6 matrix instruction on the bare codes (gemm6_kernel.h) --------------------------------
 int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noalloc) {
     g6::Params p;
@@ -258,19 +283,10 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     p.silu = a->fuse_silu != 0;
     p.gelu = a->qout != nullptr;  // the GELU is composed exactly when the next layer's input is produced (launch_impl.cuh:282-309)
 
-    // One workgroup per 128 x 256 output tile, two resident per compute unit.  A tile alone on its compute
-    // unit takes about 30 us at K = 3072 whatever else the chip does, and every part of a split tile pays for
-    // parking its sums and the last one for fetching them all: measured at K = 3072, 24 tiles take 30.9 us
-    // whole, 28.3 in two parts, 36.1 in six, 106.7 in 24; 96 tiles 31.3 whole, 31.7 in two.  So only launches
-    // that fill at most an eighth of the slots are split, and only in two.
+    // One workgroup per 128 x 256 output tile (or per part of one split along K), two resident per compute unit.
     const int mblocks = p.M_pad / g6::BM, nblocks = (p.N + g6::BN - 1) / g6::BN;
-    const int ntiles = mblocks * nblocks, kgroups = p.K / 64, slots = 2 * ncu;
-    int kparts = 1;
-    if (a->k_split > 0) {
-        kparts = a->k_split < kgroups ? a->k_split : kgroups;
-    } else if (8 * ntiles <= slots && kgroups >= 16) {
-        kparts = 2;
-    }
+    const int ntiles = mblocks * nblocks, kgroups = p.K / 64;
+    const int kparts = a->k_split > 0 ? (int)(a->k_split < kgroups ? a->k_split : kgroups) : choose_kparts(ntiles, kgroups, ncu);
     p.kparts = kparts;
     // bands of about ten row blocks, all of the same height where the count allows it
     p.band = (mblocks + (mblocks + 9) / 10 - 1) / ((mblocks + 9) / 10);

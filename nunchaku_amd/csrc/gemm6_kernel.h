@@ -314,16 +314,31 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         for (int t = 0; t < 8; t++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[t][e] = 0.f;
-        for (int pt = 0; pt < p.kparts; pt++) {
-            const __amdgpu_buffer_rsrc_t theirs = partial_rsrc(p.partials + ((size_t)tile * p.kparts + pt) * PARTIAL_SLOT_FLOATS);
+        // (two parts at a time, the requests of the next eighth of the tile in flight while this one is added;
+        // every element still adds its parts in ascending order)
+        for (int pt0 = 0; pt0 < p.kparts; pt0 += 2) {
+            const bool two = pt0 + 1 < p.kparts;
+            const __amdgpu_buffer_rsrc_t r0 = partial_rsrc(p.partials + ((size_t)tile * p.kparts + pt0) * PARTIAL_SLOT_FLOATS);
+            const __amdgpu_buffer_rsrc_t r1 = partial_rsrc(p.partials + ((size_t)tile * p.kparts + (two ? pt0 + 1 : pt0)) * PARTIAL_SLOT_FLOATS);
+            float4_t o[2][2][4];
+            auto request = [&](int t, int b) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) o[b][0][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r0, ((t * 4 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
+                if (two) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) o[b][1][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r1, ((t * 4 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
+                }
+            };
+            request(0, 0);
 #pragma unroll
             for (int t = 0; t < 8; t++) {
-                float4_t o[4];
+                if (t + 1 < 8) request(t + 1, (t + 1) & 1);
 #pragma unroll
-                for (int q = 0; q < 4; q++)
-                    o[q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(theirs, ((t * 4 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
+                for (int e = 0; e < 16; e++) acc[t][e] += o[t & 1][0][e / 4][e % 4];
+                if (two) {
 #pragma unroll
-                for (int e = 0; e < 16; e++) acc[t][e] += o[e / 4][e % 4];
+                    for (int e = 0; e < 16; e++) acc[t][e] += o[t & 1][1][e / 4][e % 4];
+                }
             }
         }
     }

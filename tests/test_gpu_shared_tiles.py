@@ -30,11 +30,11 @@ def _inputs(M_pad, K, R, seed):
 
 @pytest.mark.parametrize(
     "M,K,N,R,k_split",
-    [(256, 3072, 3072, 32, None), (256, 1024, 512, 16, 4), (512, 12288, 256, 32, 24), (300, 640, 768, 32, 10), (256, 256, 384, 16, 3), (2304, 256, 1280, 32, 2)],
+    [(256, 3072, 3072, 32, None), (512, 12288, 512, 32, None), (256, 1024, 512, 16, 4), (512, 12288, 256, 32, 24), (300, 640, 768, 32, 10), (256, 256, 384, 16, 3), (2304, 256, 1280, 32, 2)],
 )
 def test_split_tiles_match_whole_tiles(dev, M, K, N, R, k_split, monkeypatch):
     """k_split None: the library's own choice for a shape with few tiles (M = 256, K = N = 3072: 24 tiles,
-    2 parts each); 10 parts of K = 640: one k-group each; N = 384 and 1280: a ragged last column block."""
+    3 parts each; M = 512, K = 12288, N = 512: 8 tiles, 8 parts each); 10 parts of K = 640: one k-group each; N = 384 and 1280: a ragged last column block."""
     from nunchaku_amd import packing
     from nunchaku_amd.ops import gemm as gemm_mod
 
