@@ -128,8 +128,9 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * workspace per (device, stream) pair, allocated with hipMalloc the first time the pair needs it (that
  * call is not capturable into a graph and may synchronise), kept until the process ends, grown when a
  * later call needs more (after a stream synchronisation), at most 16 pairs:
- *   - INT4 with so few output tiles that they are split along K (fewer tiles than compute units, or
- *     k_split > 1): 128 KB of fp32 partial sums per tile and part;
+ *   - INT4 with so few output tiles that they are split along K (no more tiles than compute units and a long
+ *     enough K, or k_split > 1): 128 KB of fp32 partial sums per tile and part, at most 64 MB by the library's
+ *     own choice;
  *   - next_lora_down: 4 bytes per element of next_lora_act_out and 256-column block of N (128 for NVFP4) (every
  *     block leaves its share there and a small kernel launched behind the GEMM adds the shares in ascending
  *     order, so the result does not depend on the order in which the blocks finish);
