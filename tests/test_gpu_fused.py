@@ -56,7 +56,7 @@ def test_next_layer_epilogue(dev, M, K1, N1, N2, R):
     assert (la2.cpu() - want_la2).abs().max().item() <= 3e-5 * want_la2.abs().max().item() + 1e-6
 
 
-@pytest.mark.parametrize("M,K1,N1,N2,R", [(256, 256, 512, 256, 32), (150, 512, 2048, 512, 32)])
+@pytest.mark.parametrize("M,K1,N1,N2,R", [(256, 256, 512, 256, 32), (150, 512, 2048, 512, 32), (256, 3072, 512, 256, 32)])
 def test_fused_gelu_mlp(dev, M, K1, N1, N2, R):
     from nunchaku_amd.ops import fused_gelu_mlp
 
