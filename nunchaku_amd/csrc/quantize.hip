@@ -380,6 +380,10 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         // at M = 4608 the few large workgroups lose: 65 against 42).
         if (RT > 4 && p.M_pad >= 128 * 128) return launch<4, 2, 8, 1, FP4, false, true>(p, stream);
         if (RT > 2 && RT <= 4 && p.M_pad >= 256 * 64) return launch<4, 1, 4, 1, FP4, false, true>(p, stream);
+        // Up to one 16-row workgroup per compute unit (256 of them) the walk over K is what takes the time: eight waves
+        // split it (M = 256 ... 4096 at K = 3072: 7.9 ... 10.1 us against 9.0 ... 11.3 with four; K = 12288, M = 256:
+        // 19.6 against 25.5).  Beyond that two four-wave workgroups share a compute unit better (M = 4608: 14.4 against 16.2).
+        if (RT <= 2 && p.M_pad <= 4096) return launch<8, 1, 2, 1, FP4, false>(p, stream);
         if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4, false>(p, stream) : launch<4, 1, 2, 1, FP4, false>(p, stream);
         if (RT <= 4) return launch<4, 2, 4, 1, FP4, false>(p, stream);
         if (RT <= 8) return launch<4, 2, 8, 1, FP4, false>(p, stream);
