@@ -366,11 +366,29 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     if (a->k_split == 1) {  // whole tiles only: the largest workgroup count that divides the tile count
         while (ntiles % nwg != 0) nwg--;
     } else if (ntiles < ncu) {
-        // fewer tiles than compute units: several workgroups per tile, each with at least 12 units (24
-        // k-groups) of work, or K / (128 k_split) units when the caller asks for a split
+        // Fewer tiles than compute units.  A workgroup alone on its compute unit takes 1.67 us per k-group; the parties
+        // of a tile meet through the workspace, which costs the last one about 12 us + 20 us per party beyond itself
+        // (measured: 12 tiles at K = 3072, whole 80 us, two parties 72; at K = 12288 whole 290, eight parties 183; 144
+        // tiles at K = 3072 whole 85, split over all compute units 109).  So: whole tiles unless a split into equal
+        // parts pays by that count, or the caller asks for k_split parts.
+        const int kg = (int)(a->K / 64);
+        int parties = 1;
+        if (a->k_split > 1) {
+            parties = (int)a->k_split;
+        } else {
+            double best = 1.67 * kg;
+            for (int cand : {2, 3, 4, 6, 8}) {
+                if (ntiles * cand > ncu || kg / cand < 12) break;
+                const double t = 1.67 * kg / cand + 12.0 + 20.0 * (cand - 1);
+                if (t < 0.9 * best) {
+                    best = t;
+                    parties = cand;
+                }
+            }
+        }
         const long long units = (long long)ntiles * (a->K / 128);
-        const int min_units = a->k_split > 1 ? (int)((a->K / 128 + a->k_split - 1) / a->k_split) : 12;
-        long long w = units / (min_units > 0 ? min_units : 1);
+        long long w = (long long)ntiles * parties;
+        if (w > units) w = units;
         if (w > ncu) w = ncu;
         if (w > nwg) nwg = (int)w;
     }

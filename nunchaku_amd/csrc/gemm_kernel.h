@@ -327,9 +327,13 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             tile_coords(first_tile + batch0 + t, m0, n0);
             const uint32_t *sp = (const uint32_t *)p.ascales + m0 + tid;
             uint32_t mx = 0;
-            for (int g = 0; g < kgroups; g++) {
-                const uint32_t v = sp[(size_t)g * p.M_pad];
-                mx = max(max(mx, v & 0x7Fu), max((v >> 8) & 0x7Fu, max((v >> 16) & 0x7Fu, (v >> 24) & 0x7Fu)));
+            for (int g0 = 0; g0 < kgroups; g0 += 8) {  // eight requests in flight (a maximum does not mind seeing the last group again)
+                uint32_t v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = sp[(size_t)(g0 + u < kgroups ? g0 + u : kgroups - 1) * p.M_pad];
+#pragma unroll
+                for (int u = 0; u < 8; u++)
+                    mx = max(max(mx, v[u] & 0x7Fu), max((v[u] >> 8) & 0x7Fu, max((v[u] >> 16) & 0x7Fu, (v[u] >> 24) & 0x7Fu)));
             }
             int ex = 0;
             if (mx) frexpf(e4m3_to_f32(mx), &ex);  // value in [2^(ex-1), 2^ex)
