@@ -449,6 +449,10 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     const int ngroups_out = p.N / 64;
     VkSums vks;  // linear attention: the sums of the wave's two slabs
     if (NEXT && p.vk) litela_clear(vks);
+    // next layer's low-rank projection at ranks up to 32: [slab][rank tile][16-row half] sums of the wave's 128 columns,
+    // kept until both slabs are done so that the column halves meet once per tile
+    float4_t down_sums[2][2][2];
+    const bool down_once = NEXT && p.next_down && p.R_down <= 32;
     // one 32-row slab of the wave tile, instantiated twice with a compile-time slab index
     auto slab_epilogue = [&](auto MT) {
         constexpr int mt = decltype(MT)::value;
@@ -599,6 +603,13 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
                         }
                     }
                 }
+                if (down_once) {  // (one pair of rank tiles at most)
+#pragma unroll
+                    for (int g = 0; g < 2; g++)
+#pragma unroll
+                        for (int m2 = 0; m2 < 2; m2++) down_sums[mt][g][m2] = d[g][m2];
+                    break;
+                }
                 if (wn == 1) {
 #pragma unroll
                     for (int g = 0; g < 2; g++)
@@ -663,6 +674,39 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     __builtin_amdgcn_sched_barrier(0);
     slab_epilogue(std::integral_constant<int, 0>{});
     slab_epilogue(std::integral_constant<int, 1>{});
+    if (down_once) {
+        // the right column half hands its sums over through its own slab area, which it no longer needs; the left
+        // one adds and stores the workgroup's share: [32-row slab 2 wm + mt][rank tile][16-row half][64 lanes] x float4
+        static_assert(SLAB_BYTES >= 2 * 2 * 2 * 64 * 16, "a wave's sums pass through its slab area");
+        const int RT = p.R_down / 16;
+        float4_t *xchg = (float4_t *)(lds + (2 * wm + 1) * SLAB_BYTES);
+        if (wn == 1) {
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int g = 0; g < 2; g++)
+#pragma unroll
+                    for (int m2 = 0; m2 < 2; m2++) xchg[((mt * 2 + g) * 2 + m2) * 64 + lane] = down_sums[mt][g][m2];
+        }
+        __syncthreads();
+        if (wn == 0) {
+            const __amdgpu_buffer_rsrc_t slot = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(p.next_lora_part + ((size_t)nb * (p.M_pad / BM) + mb) * (size_t)(BM * p.R_down)), 0, BM * p.R_down * 4, 0x00020000);
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int g = 0; g < 2; g++) {
+                    if (g >= RT) continue;
+#pragma unroll
+                    for (int m2 = 0; m2 < 2; m2++) {
+                        const float4_t o = xchg[((mt * 2 + g) * 2 + m2) * 64 + lane], d = down_sums[mt][g][m2];
+                        const float4_t sum = float4_t{d[0] + o[0], d[1] + o[1], d[2] + o[2], d[3] + o[3]};
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), slot,
+                                                               (((((wm * 2 + mt) * RT + g) * 2 + m2) * 64) + lane) * 16, 0, 0);
+                    }
+                }
+        }
+    }
     if (NEXT && p.vk && n0 + BN > p.N / 3) {
         static_assert(SLAB_BYTES >= 2 * VK_HEAD_FLOATS * 4, "a wave's two heads pass through its slab area");
         const int third = p.N / 3;
