@@ -134,7 +134,7 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  *   - next_lora_down: 4 bytes per element of next_lora_act_out and 256-column block of N (128 for NVFP4) (every
  *     block leaves its share there and a small kernel launched behind the GEMM adds the shares in ascending
  *     order, so the result does not depend on the order in which the blocks finish);
- *   - out_vk: 4224 bytes per 32 rows and head;
+ *   - out_vk: 4224 bytes per head and 128 rows (NVFP4: 32 rows);
  *   - NVFP4 whenever the number of 256 x 256 tiles is not a multiple of the number of compute units:
  *     512 KB per compute unit.
  * Calls on one stream run in order and share the workspace safely; the same stream must not be used
