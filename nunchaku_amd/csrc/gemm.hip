@@ -363,8 +363,13 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     // persistent workgroups: one per compute unit, each walking over its share of the output tiles
     const int ntiles = (int)(a->M_pad / BM) * (int)((a->N + BN - 1) / BN);
     int nwg = ntiles < ncu ? ntiles : ncu;
-    if (a->k_split == 1) {  // whole tiles only: the largest workgroup count that divides the tile count
-        while (ntiles % nwg != 0) nwg--;
+    int divisor = nwg;  // the largest workgroup count that divides the tile count
+    while (ntiles % divisor != 0) divisor--;
+    if (a->k_split == 1 || (a->k_split == 0 && ntiles >= ncu && divisor * 100 >= ncu * 94)) {
+        // Whole tiles only: asked for, or nearly every compute unit gets a whole number of tiles anyway.  Then the
+        // workgroups that share a block of weight columns walk K in step and find it in their L2, and no sums
+        // travel through the workspace (M = 4608, N = 21504: 252 workgroups x 6 tiles 549 us, 256 even shares 560).
+        nwg = divisor;
     } else if (ntiles < ncu) {
         // Fewer tiles than compute units.  A workgroup alone on its compute unit takes 1.67 us per k-group; the parties
         // of a tile meet through the workspace, which costs the last one about 12 us + 20 us per party beyond itself
