@@ -408,6 +408,16 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     p.next_lora_part = nullptr;
     const bool next = a->qout != nullptr || a->next_lora_down != nullptr || a->rotary_emb != nullptr || a->fuse_silu || a->out_vk != nullptr;
     const bool shared_tiles = !(nwg <= ntiles && ntiles % nwg == 0);
+    p.whole_band = 0;
+    if (!shared_tiles) {
+        // bands about as high as the window of an XCD's workgroups (an eighth of them) is wide, all of the same height
+        // where the count allows it
+        const int mblocks = p.M_pad / BM;
+        int h = 1;
+        while (h * h * 8 < nwg) h++;
+        const int nbands = (mblocks + h - 1) / h;
+        p.whole_band = (mblocks + nbands - 1) / nbands;
+    }
     // every 128-column chunk's share of the next layer's low-rank projection, every row block's linear-attention sums
     const size_t share_bytes = p.next_down ? (size_t)(p.N / 128) * p.M_pad * p.R_down * 4 : 0;
     const size_t vk_bytes = p.vk ? (size_t)(p.M_pad / 32) * (p.N / 96) * VK_HEAD_FLOATS * 4 : 0;  // (this kernel: per 32-row slab)

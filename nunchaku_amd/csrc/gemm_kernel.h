@@ -115,19 +115,38 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     const int kgroups = p.K / 64, kunits = kgroups / 2;
     const int ntiles32 = p.N / 32;
     const int nwg = gridDim.x;
-    const int vwg = nwg % 8 == 0 ? ((int)blockIdx.x % 8) * (nwg / 8) + (int)blockIdx.x / 8 : (int)blockIdx.x;
+    const int xcd = (int)blockIdx.x % 8, extra = nwg % 8;  // XCD x holds nwg / 8 workgroups, one more if x < nwg % 8
+    const int vwg = xcd * (nwg / 8) + (xcd < extra ? xcd : extra) + (int)blockIdx.x / 8;
     const long long units = (long long)ntiles * kunits;
     const long long u_begin = units * vwg / nwg, u_end = units * (vwg + 1) / nwg;
     const int first_tile = (int)(u_begin / kunits);
     const int nseg = u_end > u_begin ? (int)((u_end - 1) / kunits) - first_tile + 1 : 0;
     // segment s of this workgroup: tile first_tile + s, k-groups [gb, ge)
+    // Whole tiles only (p.whole_band != 0, the workgroup count divides the tile count): in its step s workgroup v takes
+    // tile s W + v of a numbering in bands of p.whole_band row blocks, down the band first.  All workgroups walk K in
+    // step, so the 32 of an XCD, which hold consecutive numbers, cover a compact window of the output at any time and
+    // share its rows of activations and columns of weights in their L2.
     auto segment = [&](int sidx, int &tile, int &gb, int &ge) {
+        if (p.whole_band) {
+            tile = sidx * nwg + vwg;
+            gb = 0;
+            ge = kgroups;
+            return;
+        }
         tile = first_tile + sidx;
         const long long t0 = (long long)tile * kunits;
         gb = sidx == 0 ? 2 * (int)(u_begin - t0) : 0;
         ge = u_end - t0 < kunits ? 2 * (int)(u_end - t0) : kgroups;
     };
     auto tile_coords = [&](int tile, int &m0, int &n0) {
+        if (p.whole_band) {
+            const int per_band = p.whole_band * nblocks;
+            const int band = tile / per_band, in_band = tile - band * per_band;
+            const int rows = mblocks - band * p.whole_band < p.whole_band ? mblocks - band * p.whole_band : p.whole_band;
+            m0 = (band * p.whole_band + in_band % rows) * BM;
+            n0 = (in_band / rows) * BN;
+            return;
+        }
         m0 = (tile % mblocks) * BM;
         n0 = (tile / mblocks) * BN;
     };
@@ -155,7 +174,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     // follow: the segment after the one given by prev_* (the next tile, from its first k-group), without divisions
     auto make_ctx = [&](int sidx, int slot, int tid, bool follow, int prev_tile, int prev_m0, int prev_n0) {
         TileCtx c;
-        if (follow) {
+        if (follow && !p.whole_band) {
             c.tile = prev_tile + 1;
             c.gb = 0;
             const long long left = u_end - (long long)c.tile * kunits;
@@ -324,7 +343,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         // non-negative values order like unsigned bytes
         for (int t = 0; t < nbatch; t++) {
             int m0, n0;
-            tile_coords(first_tile + batch0 + t, m0, n0);
+            int tile_t, gb_t, ge_t;
+            segment(batch0 + t, tile_t, gb_t, ge_t);
+            tile_coords(tile_t, m0, n0);
             const uint32_t *sp = (const uint32_t *)p.ascales + m0 + tid;
             uint32_t mx = 0;
             for (int g0 = 0; g0 < kgroups; g0 += 8) {  // eight requests in flight (a maximum does not mind seeing the last group again)

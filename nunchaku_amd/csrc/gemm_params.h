@@ -186,6 +186,7 @@ struct GemmParams {
     // linear attention (see g6::Params) and the parked shares of the next layer's low-rank projection
     float *vk, *vk_part;
     int vk_rows;
+    int whole_band;              // 0, or (whole tiles only) the band height of the tile numbering in row blocks
     float *next_lora_part;  // [N/128 column chunks][M_pad/32 slabs][R_down/16][2][64 lanes] x float4
 };
 
