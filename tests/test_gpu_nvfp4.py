@@ -63,11 +63,12 @@ def test_nvfp4_layer_end_to_end(dev):
     check_output(y, ref.forward_quant(codes, scales, lora)[:M])
 
 
-@pytest.mark.parametrize("M,K1,N1,R", [(256, 256, 512, 16), (2304, 256, 7680, 32)])
+@pytest.mark.parametrize("M,K1,N1,R", [(256, 256, 512, 16), (2304, 256, 7680, 32), (3072, 256, 10752, 32)])
 def test_nvfp4_fused_mlp_epilogue(dev, M, K1, N1, R):
     """NVFP4 GEMM producing the next layer's NVFP4 input (no shift, signed patterns).  The second shape has 270 tiles,
     which the persistent workgroups share, and 60 column chunks whose shares of the low-rank projection are added in
-    order afterwards: the projection must be fully written (it starts as NaN) and the same from launch to launch."""
+    order afterwards: the projection must be fully written (it starts as NaN) and the same from launch to launch.  The
+    third has 504 tiles: 252 workgroups of two whole tiles each, taken in the windowed order."""
     from nunchaku_amd import packing
     from nunchaku_amd.ops import svdq_gemm_w4a4
 
