@@ -123,3 +123,26 @@ def test_mlp_flux_shape(dev):
     ref2 = make_oracle(fc2, act_unsigned=True)
     want_y = ref2.forward_quant(want_codes, want_scales, want_la2)
     check_output(y[rows], want_y)
+
+
+def test_side_streams_give_the_same_bits(dev):
+    """The library launches on the caller's current stream and keeps one workspace per (device, stream): the fused
+    MLP whose first GEMM is split along K (parked sums, arrival counters) and leaves low-rank shares, run in turn on
+    two side streams, gives what the default stream gave."""
+    from nunchaku_amd.ops import fused_gelu_mlp
+
+    M, K1, N1, N2, R = 256, 3072, 512, 256, 32
+    announce(f"fused_gelu_mlp on side streams M={M} K1={K1} N1={N1} N2={N2}")
+    fc1, fc2, x, m1, m2 = _mlp(dev, M, K1, N1, N2, R, seed=77)
+    xd = x.to(dev).view(1, M, K1)
+    want = fused_gelu_mlp(xd, m1, m2)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)]
+    outs = []
+    for s in streams + streams:
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            outs.append(fused_gelu_mlp(xd, m1, m2))
+    torch.cuda.synchronize()
+    for got in outs:
+        assert torch.equal(got, want)
