@@ -82,3 +82,38 @@ def test_noalloc_refuses_what_does_not_fit(dev, monkeypatch):
     m = make_module(synth.make_layer(c["N"], c["K"], c["R"], seed=3), dev)
     with pytest.raises(NotImplementedError, match="fixed scratch"):
         _run(dev, gemm_mod, m, **c, seed=3, no_alloc=True, k_split=16, monkeypatch=monkeypatch)
+
+
+def test_noalloc_forward_in_a_graph(dev, monkeypatch):
+    """What the entry point is for: the layer's forward (quantize, then a GEMM split along K whose parked sums and
+    arrival counters live in the fixed array) captured into a graph and replayed, with eager work of the same layer
+    between the replays; every replay gives the eager result."""
+    from nunchaku_amd.ops import gemm as gemm_mod
+
+    announce("forward through svdq_gemm_w4a4_noalloc captured into a graph")
+    monkeypatch.setattr(gemm_mod, "NO_ALLOC", True)
+    monkeypatch.setattr(gemm_mod, "K_SPLIT", None)
+    M, K, N, R = 256, 3072, 512, 32
+    m = make_module(synth.make_layer(N, K, R, seed=9), dev)
+    xs = [synth.make_activations(M, K, seed=100 + i).to(dev).view(1, M, K) for i in range(3)]
+    eager = [m(x).clone() for x in xs]
+    torch.cuda.synchronize()
+    static_x = xs[0].clone()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            m(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = m(static_x)
+    for _ in range(2):
+        for i, x in enumerate(xs):
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            z = m(x)
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager[i]) and torch.equal(z, eager[i])
