@@ -29,6 +29,18 @@ def _cases():
         opts = dict(bias=rng.random() < 0.7, scales=rng.random() < 0.4, alpha=rng.choice([1.0, 1.0, 0.5, 1.7]) if not fp4 else None,
                     lora_scales=rng.random() < 0.4, k_split=rng.choice([None, None, 1, 2, 3]) if not fp4 else rng.choice([None, 1]))
         cases.append((i, M, K, N, R, fp4, opts))
+    # long K with few tiles: the shapes where the library splits tiles along K by its own choice (INT4: in 2 to 8 parts;
+    # NVFP4: parties of equal size)
+    rng = random.Random(77)
+    for i in range(100, 112):
+        fp4 = i % 4 == 3
+        M = rng.choice([100, 256, 300, 640])
+        K = rng.choice([2048, 3072, 4096, 6144])
+        N = 128 * rng.randint(1, 8)
+        R = rng.choice([16, 32, 32, 64])
+        opts = dict(bias=rng.random() < 0.7, scales=rng.random() < 0.4, alpha=rng.choice([1.0, 0.5]) if not fp4 else None,
+                    lora_scales=rng.random() < 0.4, k_split=None)
+        cases.append((i, M, K, N, R, fp4, opts))
     return cases
 
 
