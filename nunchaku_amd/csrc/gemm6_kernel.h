@@ -145,20 +145,20 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
     // that issues its six requests back to back stands still until the memory pipeline has taken them,
     // about 30 cycles each.  First the three weight chunks (W), later the other three (R).
     auto copy_w = [&](uint32_t stage_off, int i) {  // weight chunk i of the next k-group whose weights are not requested yet
-        if (i == 0) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
-        if (i == 1) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+        if (i == 0) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory", "m0", "scc");
+        if (i == 1) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory", "m0", "scc");
         if (i == 2) {
-            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:2048" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory");
+            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3 offset:2048" :: "s"(dst_w), "s"(stage_off), "v"(copy_voff), "s"(src_w) : "memory", "m0", "scc");
             src_w += 8 * FRAG_BYTES;
         }
     };
     auto copy_r = [&](uint32_t stage_off, int i) {  // the rest: activation chunk, activation / weight-scale chunk, activation scales
-        if (i == 0) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_a), "s"(stage_off), "v"(copy_voff), "s"(src_a) : "memory");
-        if (i == 1) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_x), "s"(stage_off), "v"(copy_voff), "s"(src_x) : "memory");
+        if (i == 0) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_a), "s"(stage_off), "v"(copy_voff), "s"(src_a) : "memory", "m0", "scc");
+        if (i == 1) asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" :: "s"(dst_x), "s"(stage_off), "v"(copy_voff), "s"(src_x) : "memory", "m0", "scc");
         if (i == 2) {
             uint32_t voff4;
             asm volatile("v_lshrrev_b32 %0, 2, %1" : "=v"(voff4) : "v"(copy_voff));
-            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3" :: "s"(dst_q), "s"(stage_off), "v"(voff4), "s"(src_q) : "memory");
+            asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3" :: "s"(dst_q), "s"(stage_off), "v"(voff4), "s"(src_q) : "memory", "m0", "scc");
             src_a += 4 * FRAG_BYTES;
             src_x += stride_x;
             src_q += stride_q;

@@ -227,9 +227,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :: "s"(dst + STAGE_A + 4 * j * TILE_BYTES), "v"(voff), "s"(c.a_base[j]) : "memory");
+                         :: "s"(dst + STAGE_A + 4 * j * TILE_BYTES), "v"(voff), "s"(c.a_base[j]) : "memory", "m0");
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(voff), "s"(c.b_base[j]) : "memory");
+                         :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(voff), "s"(c.b_base[j]) : "memory", "m0");
         }
     };
     // (ordinary loads: the compiler tracks the registers they write and places the waits for them itself.
