@@ -4,12 +4,9 @@
 //
 // HBM-bound: every weight byte is read once.  The kernel reads the reference's storage as it is (no
 // repack): per 4 output rows and 64 input channels a block of 128 bytes, 32 bytes per row
-// (nunchaku/models/text_encoders/tinychat_utils.py:76-106), so a 4-row group is contiguous along K and a
-// wave-wide 16-byte load covers 4 rows x 512 channels in 1 KB.  One wave owns one 4-row group for the
-// whole K extent; lane l holds row (l % 8) / 2 and the 32 channels 512 it + 64 (l / 8) + 32 (l % 2) + [0, 32).
-// Word i2 of its 16 bytes, nibble p + 4 b, is channel 8 p + 2 i2 + b: the nibbles p and p + 4 are a pair
-// of neighbouring channels, which after dequantization is one packed bf16 pair for v_dot2_f32_bf16 against
-// the pair of activations as loaded.
+// (nunchaku/models/text_encoders/tinychat_utils.py:76-106).  Word i2 of a row's 16 bytes of a 32-channel half,
+// nibble p + 4 b, is channel 8 p + 2 i2 + b: the nibbles p and p + 4 are a pair of neighbouring channels, which
+// after dequantization is one packed bf16 pair, and the four pairs of one p are eight consecutive channels.
 #include "svdq_common.h"
 
 using namespace svdq;
@@ -26,132 +23,120 @@ struct AwqParams {
     int M, N, K;
 };
 
-typedef __bf16 bf16x2_v __attribute__((ext_vector_type(2)));
 
-// XLDS: the rows of x are copied to LDS once per workgroup (every wave needs all of x; from global memory
-// the activation loads, 64 bytes per lane, row of x and step, outweigh the weight stream from 2 rows on).
-template <int MT, bool XLDS>
-__global__ void __launch_bounds__(256) awq_gemv_kernel(AwqParams p) {
-    extern __shared__ u32x4_t xlds[];  // [M][K] bf16
+// The products go to the matrix cores (with v_dot2_f32_bf16 per row of x and pair instead, one row took 11.9 us
+// against 11.3 at K = 3072, N = 18432, four rows 17.4 against 12.0, eight 28.0 against 14.7).
+// A workgroup owns 16 output channels; its four waves take the 128-channel steps of K in turn and meet in LDS at the
+// end.  Lane l holds output channel l % 16 and the 32 input channels 128 it + 32 (l / 16) + [0, 32) of a step: the four
+// packed pairs of nibble position p (channels 8 p ... 8 p + 7 of the 32) are the second operand of the p-th
+// v_mfma_f32_16x16x32_bf16 of the step as they come, the first is x[m = l % 16][the same 8 channels] (zero for rows
+// beyond M).  The result tile has channel l % 16 and rows 4 (l / 16) + [0, 4) in lane l.
+template <bool XLDS>
+__global__ void __launch_bounds__(256) awq_gemv_mfma_kernel(AwqParams p) {
+    extern __shared__ u32x4_t xlds[];  // XLDS (x fits: up to 64 KB): [M][K] bf16; then, always, 4 waves x 64 lanes x float4
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t xquads = XLDS ? (size_t)p.M * p.K / 8 : 0;
     if (XLDS) {
-        const int n16 = p.M * p.K / 8;
-        for (int i = threadIdx.x; i < n16; i += 256) xlds[i] = ((const u32x4_t *)p.x)[i];
+        for (int i = threadIdx.x; i < (int)xquads; i += 256) xlds[i] = ((const u32x4_t *)p.x)[i];
         __syncthreads();
     }
-    // Workgroups are dealt to the 8 XCDs in turn (blockIdx % 8), each with its own L2.  A 128-byte line of
-    // scales or zeros serves 64 output rows = 16 row groups = 4 workgroups: consecutive workgroups of the
-    // row order are therefore given to the same XCD, so that the line is fetched from memory once, not 8 times.
     int wg = blockIdx.x;
-    if (gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
-    const int rg = wg * 4 + wave;  // 4-row group
-    if (rg * 4 >= p.N) return;
-    const int u = lane & 7, blk = lane >> 3;
-    const int row = rg * 4 + (u >> 1);
+    if (gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;  // neighbours in N on one XCD: they share lines of scales
+    const int n = lane & 15, kb = lane >> 4;
+    const int row_raw = wg * 16 + n;
+    const int row = row_raw < p.N ? row_raw : p.N - 1;  // a channel beyond N repeats the last one and is not stored
     const int kblocks = p.K / 64;
-    const int iters = (kblocks + 7) / 8;
-    const u32x4_t *wp = (const u32x4_t *)(p.qweight + (size_t)rg * p.K * 2) + lane;
+    const int steps = (p.K + 127) / 128;
+    const uint8_t *wrow = p.qweight + ((size_t)(row >> 2) * kblocks * 4 + (row & 3)) * 32 + (kb & 1) * 16;  // + 128 per 64-channel block
+    const bool xrow = n < p.M;  // this lane supplies row n of x to the first operand
 
-    float acc[MT];
-#pragma unroll
-    for (int m = 0; m < MT; m++) acc[m] = 0.f;
-
-    // Weights, scales and zeros are requested DEPTH steps ahead (a ring of DEPTH + 1 register sets, indexed
-    // statically).  Every request is unconditional: a step or channel block past the end re-reads the last
-    // valid one and gets scale and zero 0, so that it contributes nothing; a request behind a branch would make
-    // the compiler's wait counting assume the worst and wait for the requests made ahead.
     constexpr int DEPTH = 3;
     u32x4_t wq[DEPTH + 1];
     uint16_t sq[DEPTH + 1], zq[DEPTH + 1];
-    auto load_w = [&](int it, int slot) {
-        int kb = it * 8 + blk;
-        kb = kb < kblocks ? kb : kblocks - 1;
-        wq[slot] = __builtin_nontemporal_load((const u32x4_t *)(p.qweight + ((size_t)rg * kblocks + kb) * 128) + u);
-        sq[slot] = p.scales[(size_t)kb * p.N + row];
-        zq[slot] = p.zeros[(size_t)kb * p.N + row];
+    auto block_of = [&](int it) {  // the lane's 64-channel block in step it, clamped to the last valid one
+        const int cb = it * 2 + (kb >> 1);
+        return cb < kblocks ? cb : kblocks - 1;
     };
+    auto load_w = [&](int it, int slot) {
+        const int cb = block_of(it);
+        wq[slot] = __builtin_nontemporal_load((const u32x4_t *)(wrow + (size_t)cb * 128));
+        sq[slot] = p.scales[(size_t)cb * p.N + row];
+        zq[slot] = p.zeros[(size_t)cb * p.N + row];
+    };
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
     auto step = [&](int it, int slot) {
-        const bool ok = it * 8 + blk < kblocks;
+        const bool ok = it * 2 + (kb >> 1) < kblocks;
         const u32x4_t w = wq[slot];
         const float s = ok ? bf16_bits_to_f32(sq[slot]) : 0.f, z = ok ? bf16_bits_to_f32(zq[slot]) : 0.f;
-        load_w(it + DEPTH, slot == 0 ? DEPTH : slot - 1);  // the set freed by the previous step ... see the ring below
-        // activations of this lane's 32 channels for every row of x (a channel block past the end is
-        // clamped to the last one: its weights are zero)
-        int kb = it * 8 + blk;
-        kb = kb < kblocks ? kb : kblocks - 1;
-        const int k0 = kb * 64 + 32 * (u & 1);
-        uint32_t xv[MT][16];
+        load_w(it + 4 * DEPTH, slot == 0 ? DEPTH : slot - 1);
+        const int k0 = block_of(it) * 64 + 32 * (kb & 1);
+        u32x4_t xa[4];
 #pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const size_t xoff = (size_t)(m < p.M ? m : p.M - 1) * p.K + k0;
-            const u32x4_t *xp = XLDS ? xlds + xoff / 8 : (const u32x4_t *)(p.x + xoff);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const u32x4_t v = xp[i];
-                xv[m][4 * i] = v[0]; xv[m][4 * i + 1] = v[1]; xv[m][4 * i + 2] = v[2]; xv[m][4 * i + 3] = v[3];
+        for (int j = 0; j < 4; j++) {
+            xa[j] = u32x4_t{0, 0, 0, 0};
+            if (xrow) {
+                const size_t xoff = (size_t)n * p.K + k0 + 8 * j;
+                xa[j] = XLDS ? xlds[xoff / 8] : *(const u32x4_t *)(p.x + xoff);
             }
         }
+        const uint32_t lo[4] = {w[0] & 0x0F0F0F0Fu, w[1] & 0x0F0F0F0Fu, w[2] & 0x0F0F0F0Fu, w[3] & 0x0F0F0F0Fu};
+        const uint32_t hi[4] = {(w[0] >> 4) & 0x0F0F0F0Fu, (w[1] >> 4) & 0x0F0F0F0Fu, (w[2] >> 4) & 0x0F0F0F0Fu, (w[3] >> 4) & 0x0F0F0F0Fu};
 #pragma unroll
-        for (int i2 = 0; i2 < 4; i2++) {
-            const uint32_t lo = w[i2] & 0x0F0F0F0Fu, hi = (w[i2] >> 4) & 0x0F0F0F0Fu;  // nibbles 0 2 4 6 / 1 3 5 7, one per byte
+        for (int pq = 0; pq < 4; pq++) {
+            // nibbles pq and pq + 4 of word i2 are channels 8 pq + 2 i2 and 8 pq + 2 i2 + 1
+            u32x4_t wb;
 #pragma unroll
-            for (int pq = 0; pq < 4; pq++) {
-                const uint32_t src = (pq & 1) ? hi : lo;
-                const int byte = pq >> 1;  // nibble pq is byte pq / 2 of its word, nibble pq + 4 two bytes higher
+            for (int i2 = 0; i2 < 4; i2++) {
+                const uint32_t src = (pq & 1) ? hi[i2] : lo[i2];
+                const int byte = pq >> 1;
                 const float q0 = (float)((src >> (8 * byte)) & 0xFFu), q1 = (float)((src >> (8 * byte + 16)) & 0xFFu);
-                // bf16(code * scale + zero): the sum of a 12-bit product and an 8-bit number, rounded once to fp32
-                // and then to bf16 (the reference rounds once, to bf16; the two differ only on exact ties of the
-                // second rounding)
-                const uint32_t pair = pack_bf16x2(__builtin_fmaf(q0, s, z), __builtin_fmaf(q1, s, z));
-                const int xw = i2 + 4 * pq;  // channels 8 pq + 2 i2 + {0, 1} = word 4 pq + i2 of the lane's 16
-#pragma unroll
-                for (int m = 0; m < MT; m++)
-                    acc[m] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, pair), __builtin_bit_cast(bf16x2_v, xv[m][xw]), acc[m], false);
+                wb[i2] = pack_bf16x2(__builtin_fmaf(q0, s, z), __builtin_fmaf(q1, s, z));  // bf16(code * scale + zero), see above
             }
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xa[pq]), __builtin_bit_cast(bf16x8_t, wb), acc, 0, 0, 0);
         }
     };
+    // wave w takes the steps w, w + 4, ...; the ring of DEPTH + 1 register sets is indexed statically
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) load_w(d, d);
-    // step it uses set it % (DEPTH + 1) and refills the set of step it - 1, which is (it + DEPTH) % (DEPTH + 1)
-    for (int it0 = 0; it0 < iters; it0 += DEPTH + 1) {
+    for (int d = 0; d < DEPTH; d++) load_w(wave + 4 * d, d);
+    for (int it0 = wave; it0 < steps; it0 += 4 * (DEPTH + 1)) {
 #pragma unroll
         for (int sl = 0; sl <= DEPTH; sl++) {
-            if (it0 + sl >= iters) goto done;
-            step(it0 + sl, sl);
+            if (it0 + 4 * sl >= steps) goto done;
+            step(it0 + 4 * sl, sl);
         }
     }
 done:
-    // lanes with the same (l % 8) / 2 hold parts of the same row
+    float4_t *red = (float4_t *)(xlds + xquads);
+    red[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+        const float4_t a1 = red[64 + lane], a2 = red[128 + lane], a3 = red[192 + lane];
 #pragma unroll
-    for (int m = 0; m < MT; m++) {
-        float a = acc[m];
-        a += __shfl_xor(a, 1);
-        a += __shfl_xor(a, 8);
-        a += __shfl_xor(a, 16);
-        a += __shfl_xor(a, 32);
-        if (lane < 8 && (lane & 1) == 0 && m < p.M) {
-            // the reference stores bf16 and adds the bias to that (linear.py:183-185): two roundings
-            float o = bf16_bits_to_f32(f32_to_bf16_bits(a));
-            if (p.bias) o = bf16_bits_to_f32(f32_to_bf16_bits(o + bf16_bits_to_f32(p.bias[row])));
-            p.out[(size_t)m * p.N + row] = (uint16_t)f32_to_bf16_bits(o);
+        for (int i = 0; i < 4; i++) {
+            const int m = 4 * kb + i;
+            if (m < p.M && row_raw < p.N) {
+                // the reference stores bf16 and adds the bias to that (linear.py:183-185): two roundings
+                float o = bf16_bits_to_f32(f32_to_bf16_bits(((acc[i] + a1[i]) + a2[i]) + a3[i]));
+                if (p.bias) o = bf16_bits_to_f32(f32_to_bf16_bits(o + bf16_bits_to_f32(p.bias[row])));
+                p.out[(size_t)m * p.N + row] = (uint16_t)f32_to_bf16_bits(o);
+            }
         }
     }
 }
 
-template <int MT>
-int launch(const AwqParams &p, hipStream_t stream) {
-    const size_t xbytes = (size_t)p.M * p.K * 2;
-    const dim3 grid((p.N / 4 + 3) / 4);
+int launch_mfma(const AwqParams &p, hipStream_t stream) {
+    const size_t xbytes = (size_t)p.M * p.K * 2, red = 4 * 64 * 16;
+    const dim3 grid((p.N + 15) / 16);
     if (xbytes <= 64 * 1024) {
-        auto kern = awq_gemv_kernel<MT, true>;
-        if (xbytes > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)xbytes);
-            if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "awq_gemv: cannot reserve %zu bytes of LDS: %s", xbytes, hipGetErrorString(e));
+        auto kern = awq_gemv_mfma_kernel<true>;
+        if (xbytes + red > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(xbytes + red));
+            if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "awq_gemv: cannot reserve %zu bytes of LDS: %s", xbytes + red, hipGetErrorString(e));
         }
-        hipLaunchKernelGGL(kern, grid, dim3(256), xbytes, stream, p);
+        hipLaunchKernelGGL(kern, grid, dim3(256), xbytes + red, stream, p);
     } else {
-        hipLaunchKernelGGL((awq_gemv_kernel<MT, false>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((awq_gemv_mfma_kernel<false>), grid, dim3(256), red, stream, p);
     }
     return check_launch("awq_gemv_w4a16");
 }
@@ -170,8 +155,5 @@ extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *a, void *stream) {
     AwqParams p{(const uint16_t *)a->x, (const uint8_t *)a->qweight, (const uint16_t *)a->scales, (const uint16_t *)a->zeros,
                 (const uint16_t *)a->bias, (uint16_t *)a->out, (int)a->M, (int)a->N, (int)a->K};
     hipStream_t st = (hipStream_t)stream;
-    if (a->M == 1) return launch<1>(p, st);
-    if (a->M == 2) return launch<2>(p, st);
-    if (a->M <= 4) return launch<4>(p, st);
-    return launch<8>(p, st);
+    return launch_mfma(p, st);
 }
