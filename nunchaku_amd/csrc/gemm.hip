@@ -365,8 +365,9 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     int nwg = ntiles < ncu ? ntiles : ncu;
     int divisor = nwg;  // the largest workgroup count that divides the tile count
     while (ntiles % divisor != 0) divisor--;
-    if (a->k_split == 1 || (a->k_split == 0 && ntiles >= ncu && divisor * 100 >= ncu * 94)) {
-        // Whole tiles only: asked for, or nearly every compute unit gets a whole number of tiles anyway.  Then the
+    if (a->k_split == 1 || (a->k_split == 0 && ntiles >= ncu && divisor * 100 >= ncu * 84)) {
+        // Whole tiles only: asked for, or at least 84 % of the compute units get a whole number of tiles (M = 4608,
+        // N = 9216: 216 workgroups x 3 tiles 257 us, 256 even shares 256).  Then the
         // workgroups that share a block of weight columns walk K in step and find it in their L2, and no sums
         // travel through the workspace (M = 4608, N = 21504: 252 workgroups x 6 tiles 549 us, 256 even shares 560).
         nwg = divisor;

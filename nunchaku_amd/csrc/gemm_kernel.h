@@ -375,46 +375,12 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
    for (int ti = 0; ti < nbatch; ti++) {
     const bool have_next = ti + 1 < nbatch;
     refresh_thread_coordinates();
-    // A tile shared with the next workgroup (this one holds its first k-groups, the neighbour the rest):
-    // the neighbour works on it first thing, so its partial sums are normally parked in the workspace by
-    // now.  Then they are the initial value of the accumulators and this workgroup runs the epilogue.
-    // Slots of the workspace: workgroup v parks the tile its share begins in at 2 v, the one it ends in
-    // at 2 v + 1; layout of a slot [64 quads][256 threads] x float4 (a wave's access covers 1 KB).
-    bool preloaded = false;
-    bool two_parties = false;
-    if (cur.gb == 0 && cur.ge != kgroups) {
-        int lo, hi;
-        tile_parties(cur.tile, lo, hi);
-        two_parties = hi - lo == 1;
-    }
-    if (two_parties) {
-        int *flag = (int *)(lds + FLAG_OFF);
-        if (tid == 0) *flag = __hip_atomic_load(p.counters + cur.tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        preloaded = *flag != 0;
-        __syncthreads();
-    }
-    if (preloaded) {
-        const __amdgpu_buffer_rsrc_t theirs_rsrc = partial_rsrc((const float4_t *)p.partials + (size_t)(2 * vwg + 2) * (64 * 256));
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float4_t o[16];
+    for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int k = 0; k < 16; k++) o[k] = load_partial(theirs_rsrc, tid, i * 16 + k);
+        for (int j = 0; j < 4; j++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) acc[i][j][e] = o[j * 4 + e / 4][e % 4];
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), stated in a way the compiler's bookkeeping understands
-    } else {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-    }
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     read_raw(0, araw, braw, asc, bsc);
     SVDQ_CONVERT(araw, braw, asc, bsc, 0, a0, b0)
@@ -458,17 +424,17 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     if (have_next) nxt = make_ctx(batch0 + ti + 1, ti + 1, tid, true, cur.tile, cur.m0, cur.n0);
 
     // ---- a tile shared with other workgroups ---------------------------------------------------
-    // Every party holds the sum over its part of K.  Whoever finishes last adds the others' partial sums
-    // (fp32; with two parties the result does not depend on who that is, with more the order of the
-    // additions is fixed: ascending workgroup, own sums last) and runs the epilogue.  Nobody waits: the
-    // others park their accumulators in their slot of the workspace and go on.
+    // Every party holds the sum over its part of K.  Whoever finishes last adds all parties' sums in ascending order
+    // of the workgroups, its own (from its registers) in their place: the result does not depend on who that is, so
+    // the output is the same from launch to launch.  Nobody waits: the others park their accumulators in their slot
+    // of the workspace (workgroup v parks the tile its share begins in at 2 v, the one it ends in at 2 v + 1; layout of
+    // a slot [64 quads][256 threads] x float4, a wave's access covers 1 KB) and go on.  (Starting the accumulators
+    // from a neighbour's parked sums where they happen to be there already saves the parking, but changes the order
+    // of the additions with the timing: outputs then differed in their last bit from launch to launch.)
     bool run_epilogue = true, combine = false;
     int party_lo = 0, party_hi = -1;  // (worked out here, not ahead of the main loop, where they would occupy registers)
-    if (!preloaded && (cur.gb != 0 || cur.ge != kgroups)) tile_parties(tile_e, party_lo, party_hi);
-    if (preloaded) {
-        // the neighbour's sums were the initial value; leave the counter at zero for the next launch
-        if (tid == 0) __hip_atomic_store(p.counters + cur.tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else if (cur.gb != 0 || cur.ge != kgroups) {
+    if (cur.gb != 0 || cur.ge != kgroups) {
+        tile_parties(tile_e, party_lo, party_hi);
         const bool is_head = cur.gb != 0;  // the share begins inside this tile
         const int others = party_hi - party_lo;
         float4_t *mine = (float4_t *)p.partials + (size_t)(2 * vwg + (is_head ? 0 : 1)) * (64 * 256);
@@ -632,12 +598,18 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         const float rn = ldexpf(1.0f, -tile_shift[wm * 128 + mt * 32 + r32]);
         // (the accumulators are only read from here on: updating them in place makes the register
         // allocator copy and spill whole tuples)
-        float4_t other[16];
+        float4_t other[16];  // COMBINE: the parties' sums of this slab, added in ascending order of the workgroups
         if (COMBINE) {
 #pragma unroll
             for (int k = 0; k < 16; k++) other[k] = float4_t{0.f, 0.f, 0.f, 0.f};
             for (int v = party_lo; v <= party_hi; v++) {
-                if (v == vwg) continue;
+                if (v == vwg) {
+#pragma unroll
+                    for (int k = 0; k < 16; k++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) other[k][i] += acc[mt][k >> 2][4 * (k & 3) + i];
+                    continue;
+                }
                 // a workgroup parks the tile its share begins inside at slot 2 v, otherwise at 2 v + 1
                 const bool begins_inside = units * v / nwg > (long long)tile_e * kunits;
                 const __amdgpu_buffer_rsrc_t r = partial_rsrc((const float4_t *)p.partials + (size_t)(2 * v + (begins_inside ? 0 : 1)) * (64 * 256));
@@ -667,7 +639,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
                 if (COMBINE) {
                     const float4_t o = other[nt * 4 + q];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf((acc[mt][nt][4 * q + i] + o[i]) * rn, cf[i], bs[i]);
+                    for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf(o[i] * rn, cf[i], bs[i]);
                 } else {
 #pragma unroll
                     for (int i = 0; i < 4; i++) v[nt][4 * q + i] = __builtin_fmaf(acc[mt][nt][4 * q + i] * rn, cf[i], bs[i]);

@@ -91,10 +91,12 @@ def test_nvfp4_fused_mlp_epilogue(dev, M, K1, N1, R):
         torch.cuda.synchronize()
 
     run()
-    first = la2.clone()
-    for _ in range(2):
+    first, first_out, first_codes = la2.clone(), out.clone(), qout.clone()
+    for _ in range(6):
         la2.fill_(float("nan"))
         run()
+        # (which of a shared tile's workgroups finishes last changes from launch to launch; the sums must not)
+        assert torch.equal(out, first_out) and torch.equal(qout, first_codes), "the output changed between two launches"
         assert torch.equal(la2, first), "the next layer's low-rank input changed between two launches"
     h = out.cpu()
     want_codes, want_scales = quant.quantize_act_nvfp4(h, fc2.smooth)
