@@ -181,3 +181,35 @@ def test_forward_refuses_a_parameter_of_the_wrong_shape(dev):
     m.proj_up = torch.nn.Parameter(m.proj_up.data[:128].clone(), requires_grad=False)
     with pytest.raises(ValueError):
         m(x)
+
+
+def test_one_layer_from_two_threads(dev):
+    """A layer's prepared argument blocks are shared by the threads that call it: each call fills them and launches
+    under the layer's lock, so concurrent forwards with different row counts give what they give alone."""
+    import threading
+
+    announce("one layer called from two threads")
+    layer = synth.make_layer(384, 3072, 32, seed=35)  # (K = 3072 with few tiles: the GEMM takes the split path and its workspace)
+    m = make_module(layer, dev)
+    xs = {rows: synth.make_activations(rows, 3072, seed=rows).to(dev).view(1, rows, 3072) for rows in (100, 300)}
+    want = {rows: m(x).clone() for rows, x in xs.items()}
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(rows):
+        try:
+            for _ in range(50):
+                y = m(xs[rows])
+                torch.cuda.synchronize()
+                if not torch.equal(y, want[rows]):
+                    errors.append(f"rows={rows}: a forward differs")
+                    return
+        except Exception as e:  # (an exception in a thread would otherwise pass unnoticed)
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=work, args=(rows,)) for rows in xs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
