@@ -15,8 +15,10 @@ Arithmetic: ``w = bf16(code * scale + zero)`` (one rounding: ``__hfma2``, gemv_a
 stored tensor, i.e. minus the scaled zero point, tinychat_utils.py:187), ``out[m, n] = sum_k w[n, k] x[m, k]``
 accumulated in fp32.  The reference rounds every product to bf16 first (``__hmul2``, gemv_awq.cu:197);
 that is a loss of the reference's, not part of the definition: ``round_products=True`` reproduces it to
-size the difference.  Parity status: no fixture of the reference covers this path (unpinned by reference
-fixtures); the layout is pinned by the two derivations, the arithmetic by the library matmul.
+size the difference.  Parity status: the storage order and the scale / zero convention are pinned by golden vectors
+written by the reference's own ``pack_w4`` and ``convert_to_tinychat_w4x16y16_linear_weight``
+(tests/golden/awq_vectors.npz) and by the two derivations, the arithmetic by the library matmul; the reference holds
+no output fixture of the GEMV kernel itself.
 """
 
 from __future__ import annotations

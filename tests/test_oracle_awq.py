@@ -45,3 +45,29 @@ def test_gemv_against_library_matmul_and_product_rounding_is_small():
     lossy = awq.gemv(x, codes, scales, zeros, round_products=True)
     rel = ((lossy - got).norm() / got.norm()).item()
     assert rel < 5e-3  # the reference's bf16 products: a loss of a few 1e-4, not part of the definition
+
+
+def test_against_the_reference_packer_and_converter():
+    """Golden vectors written by the reference's own ``pack_w4`` and ``convert_to_tinychat_w4x16y16_linear_weight``
+    (tests/golden/make_awq_vectors.py): the storage order of the codes, and the convention that the stored zero is
+    minus the weight-unit zero point, so that ``code * scale + zero`` gives the weight back."""
+    from pathlib import Path
+
+    v = np.load(Path(__file__).parent / "golden" / "awq_vectors.npz")
+    codes = v["codes"].astype(np.int64)
+    oc, ic = codes.shape
+    assert np.array_equal(awq.pack_w4(codes), v["packed"])
+    assert np.array_equal(awq.unpack_w4(v["packed"]), codes)
+    # the converter: a weight that is exactly (code - zero_point) * scale comes back as the same codes ...
+    assert np.array_equal(awq.unpack_w4(v["qweight"]), codes)
+    ng = ic // 64
+    scale = torch.from_numpy(v["scale_bits"]).view(torch.bfloat16)  # [oc, ng]
+    qscale = torch.from_numpy(v["qscale_bits"]).view(torch.bfloat16)  # [padded groups, oc]
+    qzero = torch.from_numpy(v["qzero_bits"]).view(torch.bfloat16)
+    assert torch.equal(qscale[:ng], scale.t())
+    assert torch.equal(qzero[:ng].float(), -(torch.from_numpy(v["zero_point"]).float() * scale.float()).t())
+    assert not qscale[ng:].any() and not qzero[ng:].any()
+    # ... and the oracle's dequantization of what the converter stored is the weight, bit for bit
+    w = torch.from_numpy(v["weight_bits"]).view(torch.bfloat16)
+    got = awq.dequant(torch.from_numpy(codes), qscale[:ng], qzero[:ng])
+    assert torch.equal(got.view(torch.int16), w.view(torch.int16))
