@@ -39,7 +39,7 @@ extern "C" {
 #define SVDQ_EUNSUPPORTED -2 /* valid request that this build does not implement */
 #define SVDQ_ELAUNCH -3      /* the HIP runtime refused the launch */
 
-#define SVDQ_ABI_VERSION 4
+#define SVDQ_ABI_VERSION 5
 
 int svdq_abi_version(void);
 const char *svdq_last_error(void);
@@ -104,7 +104,8 @@ typedef struct svdq_quantize_args {
     const void *lora_down;  /* native proj_down (svdq_repack_lora_down) or NULL when R == 0       */
     float *lora_act_out;    /* fp32 [M_pad, R] row-major; fully written (no pre-zero needed)       */
     const float *smooth_rcp;/* fp32 [K] from svdq_repack_smooth, or NULL for no smoothing          */
-    int64_t M, M_pad, K, R;
+    int64_t M, M_pad, K, R; /* R: a multiple of 16 up to 1024; above 128 the projection takes one more
+                               launch over x per 128 ranks                                          */
     int32_t fp4;            /* 0: INT4 group 64 (signed); 1: NVFP4 group 16                        */
     int32_t fuse_glu;       /* 1: input is bf16 [M, 2K], pairs (value, gate); the K columns that are
                                quantized and projected are bf16(value * bf16(gate * sigmoid(gate)))
@@ -125,9 +126,7 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  * fp16 matrix instruction with dequantized operands (persistent workgroups, 256 x 256 tiles).
  *
  * Workspace.  Most INT4 calls need none and touch no global state.  Four kinds of call keep a
- * workspace per (device, stream) pair, allocated with hipMalloc the first time the pair needs it (that
- * call is not capturable into a graph and may synchronise), kept until the process ends, grown when a
- * later call needs more (after a stream synchronisation), at most 16 pairs:
+ * workspace per (device, stream) pair, allocated with hipMalloc the first time the pair needs it:
  *   - INT4 with so few output tiles that they are split along K (no more tiles than compute units and a long
  *     enough K, or k_split > 1): 128 KB of fp32 partial sums per tile and part, at most 64 MB by the library's
  *     own choice;
@@ -137,8 +136,16 @@ int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *args, void *strea
  *   - out_vk: 4224 bytes per head and 128 rows (NVFP4: 32 rows);
  *   - NVFP4 whenever the number of 256 x 256 tiles is not a multiple of the number of compute units:
  *     512 KB per compute unit.
+ * A block that a launch has used is never freed or moved by a later call: a HIP graph that captured a call keeps
+ * the block's address.  A pair that comes to need more gets a new block at least half as large again and the old
+ * one stays allocated (all the blocks a pair has outgrown are smaller than twice its present one); nothing
+ * synchronises.  svdq_release_workspaces frees them all.  A call that would have to allocate while its stream is
+ * being captured returns SVDQ_EUNSUPPORTED: make the call once before the capture (the block is then there), or
+ * use svdq_gemm_w4a4_noalloc, the variant for callers that cannot allocate.
  * Calls on one stream run in order and share the workspace safely; the same stream must not be used
- * from two threads at once.  svdq_gemm_w4a4_noalloc is the variant for callers that cannot allocate.
+ * from two threads at once.
+ *
+ * Ranks: R_up and R_down are multiples of 16 up to 1024 (the reference's MAX_RANK, lora.cuh:22).
  * ------------------------------------------------------------------------------------------ */
 typedef struct svdq_gemm_args {
     const void *act;        /* as written by operator 1 (INT4: E2M3 fragments; NVFP4: nibble tiles)     */
@@ -226,6 +233,12 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
  * in time on one GPU race with each other.  What a launch needs to be zero at its start is cleared by a
  * fill kernel on `stream` first. */
 int svdq_gemm_w4a4_noalloc(const svdq_gemm_args *args, void *stream);
+
+/* Frees every workspace block svdq_gemm_w4a4 has allocated, on all devices, after waiting for the work
+ * enqueued on them (hipDeviceSynchronize).  No counterpart in the reference (which allocates per call
+ * through its tensor type).  The caller promises that no other thread is inside svdq_gemm_w4a4 and that no
+ * HIP graph that captured a call of it will be replayed afterwards.  Later calls allocate again. */
+int svdq_release_workspaces(void);
 
 /* ------------------------------------------------------------------------------------------
  * Linear attention, second half: q[b][t][h][:] <- (vk[b][h][:32] q) / (vk[b][h][32] . q + eps), in place.

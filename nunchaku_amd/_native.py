@@ -24,13 +24,13 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
-SVDQ_ABI_VERSION = 4
+SVDQ_ABI_VERSION = 5
 EXPORTED_SYMBOLS = [
     "svdq_abi_version", "svdq_last_error",
     "svdq_repack_qweight", "svdq_repack_wscales", "svdq_repack_wmscales", "svdq_repack_vector",
     "svdq_repack_smooth", "svdq_repack_lora_down", "svdq_repack_lora_up", "svdq_repack_rotemb",
     "svdq_quantize_w4a4_act_fuse_lora", "svdq_gemm_w4a4", "svdq_gemm_w4a4_noalloc", "svdq_awq_gemv_w4a16",
-    "svdq_linearattn_vk_mul_q",
+    "svdq_linearattn_vk_mul_q", "svdq_release_workspaces",
 ]
 
 
@@ -143,6 +143,7 @@ def lib() -> ctypes.CDLL:
         L.svdq_gemm_w4a4_noalloc.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), vp]
         L.svdq_linearattn_vk_mul_q.argtypes = [vp, vp, i64, i64, i64, i64, ctypes.c_float, vp]
+        L.svdq_release_workspaces.argtypes = []
         for name in EXPORTED_SYMBOLS:
             getattr(L, name)
             if name not in ("svdq_last_error",):

@@ -134,9 +134,9 @@ int launch_mfma(const AwqParams &p, hipStream_t stream) {
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(xbytes + red));
             if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "awq_gemv: cannot reserve %zu bytes of LDS: %s", xbytes + red, hipGetErrorString(e));
         }
-        hipLaunchKernelGGL(kern, grid, dim3(256), xbytes + red, stream, p);
+        SVDQ_LAUNCH(kern, grid, dim3(256), xbytes + red, stream, p);
     } else {
-        hipLaunchKernelGGL((awq_gemv_mfma_kernel<false>), grid, dim3(256), red, stream, p);
+        SVDQ_LAUNCH((awq_gemv_mfma_kernel<false>), grid, dim3(256), red, stream, p);
     }
     return check_launch("awq_gemv_w4a16");
 }

@@ -15,13 +15,18 @@ int launch_next(const Params &p, int nwg, hipStream_t stream);
 
 #include <mutex>
 #include <stdlib.h>
+#include <vector>
 
 namespace {
 // Workspace of one (device, stream) pair: launches on one stream run one after the other and can share
 // it, launches on different streams may overlap and must not.  It is allocated the first time a launch
-// needs one and kept until the process ends.  The first `zero_bytes` hold arrival counters: zero when
-// allocated, and every launch that completes leaves them at zero again.  The rest is scratch (parked
-// partial sums, low-rank shares).
+// needs one.  A block that has been handed to a launch is never freed behind the caller's back: a HIP graph
+// captured through this entry point holds the block's address for as long as the graph lives.  A pair
+// that needs more than it has gets a new, larger block (at least half as large again, so that all the
+// blocks a pair ever outgrew stay below twice its present one) and the old one is retired, still
+// allocated; svdq_release_workspaces is the only place that frees.  The first `zero_bytes` hold arrival
+// counters: zero when allocated, and every launch that completes leaves them at zero again.  The rest is
+// scratch (parked partial sums, low-rank shares).
 struct Workspace {
     int dev;
     hipStream_t stream;
@@ -29,9 +34,12 @@ struct Workspace {
     size_t zero_bytes, scratch_bytes;
     bool dirty;  // a launch failed: the zero region is cleared again before the next use
 };
-constexpr int MAX_WORKSPACES = 16;
-Workspace g_ws[MAX_WORKSPACES];
-int g_ws_count = 0;
+struct Retired {
+    int dev;
+    void *ptr;
+};
+std::vector<Workspace> g_ws;
+std::vector<Retired> g_retired;
 std::mutex g_ws_mutex;  // held from the look-up until the launch that uses the workspace has been enqueued
 
 __global__ void zero_f32_kernel(float *p, int64_t n) {
@@ -105,46 +113,49 @@ __global__ void __launch_bounds__(256) reduce_vk_kernel(const float *part, float
 
 void clear_zero_region(Workspace *w) {
     const int64_t n = (int64_t)(w->zero_bytes / 4);
-    if (n > 0) hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, w->stream, (float *)w->ptr, n);
+    if (n > 0) SVDQ_LAUNCH(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, w->stream, (float *)w->ptr, n);
     w->dirty = false;
 }
 
 // (the caller holds g_ws_mutex) returns nullptr, with the error text set, on failure
 Workspace *get_workspace(int dev, hipStream_t stream, size_t zero_bytes, size_t scratch_bytes) {
     Workspace *w = nullptr;
-    for (int i = 0; i < g_ws_count; i++)
-        if (g_ws[i].dev == dev && g_ws[i].stream == stream) w = &g_ws[i];
+    for (Workspace &cand : g_ws)
+        if (cand.dev == dev && cand.stream == stream) w = &cand;
     if (w && w->zero_bytes >= zero_bytes && w->scratch_bytes >= scratch_bytes) {
         if (w->dirty) clear_zero_region(w);
         return w;
     }
-    if (!w) {
-        if (g_ws_count == MAX_WORKSPACES) {
-            fail(SVDQ_ELAUNCH, "gemm: more than %d (device, stream) pairs need a workspace", MAX_WORKSPACES);
-            return nullptr;
-        }
-        w = &g_ws[g_ws_count];
-        *w = Workspace{dev, stream, nullptr, 0, 0, false};
-    } else {
-        // grow: earlier launches on this stream may still be using the old block
-        (void)hipStreamSynchronize(stream);
-        (void)hipFree(w->ptr);
-        w->ptr = nullptr;
+    // A new block is needed.  Not while the stream is being captured: the allocation is not a stream
+    // operation, and the runtime refuses it in a capture of the global mode.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone) {
+        fail(SVDQ_EUNSUPPORTED, "gemm: this call needs %zu bytes of workspace that the stream's pair does not have yet, and the stream is being "
+             "captured: make the call once before the capture, or use svdq_gemm_w4a4_noalloc", zero_bytes + scratch_bytes);
+        return nullptr;
+    }
+    if (w) {
         if (zero_bytes < w->zero_bytes) zero_bytes = w->zero_bytes;
-        if (scratch_bytes < w->scratch_bytes) scratch_bytes = w->scratch_bytes;
-        w->zero_bytes = w->scratch_bytes = 0;
+        if (scratch_bytes < w->scratch_bytes + w->scratch_bytes / 2) scratch_bytes = w->scratch_bytes + w->scratch_bytes / 2;
     }
     zero_bytes = (zero_bytes + (1u << 20) - 1) & ~(size_t)((1u << 20) - 1);  // in steps of 1 MB: few regrows
     uint8_t *ptr = nullptr;
     hipError_t e = hipMalloc((void **)&ptr, zero_bytes + scratch_bytes);
     if (e != hipSuccess) {
+        (void)hipGetLastError();
         fail(SVDQ_ELAUNCH, "gemm: cannot allocate %zu bytes of workspace: %s", zero_bytes + scratch_bytes, hipGetErrorString(e));
         return nullptr;
+    }
+    if (w) {
+        // launches already enqueued on this stream (and graphs that captured this block) go on using the old block
+        g_retired.push_back(Retired{dev, w->ptr});
+    } else {
+        g_ws.push_back(Workspace{dev, stream, nullptr, 0, 0, false});
+        w = &g_ws.back();
     }
     w->ptr = ptr;
     w->zero_bytes = zero_bytes;
     w->scratch_bytes = scratch_bytes;
-    if (w == &g_ws[g_ws_count]) g_ws_count++;
     clear_zero_region(w);  // on the caller's stream: ordered before the launch that follows
     return w;
 }
@@ -203,7 +214,7 @@ bool acquire_workspace(bool noalloc, int dev, hipStream_t st, size_t zero_bytes,
     // zero, one that failed or was aborted does not: what this launch needs to be zero is cleared (by a
     // fill kernel, which a caller's graph capture can record).
     const int64_t n = (int64_t)((zero_bytes + 15) / 16 * 4);
-    if (n > 0) hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, (float *)base, n);
+    if (n > 0) SVDQ_LAUNCH(zero_f32_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, (float *)base, n);
     *v = WorkspaceView{base, base + NOALLOC_ZERO_BYTES, nullptr};
     return true;
 }
@@ -268,7 +279,7 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     p.M_pad = (int)a->M_pad; p.N = (int)a->N; p.K = (int)a->K;
     p.M_out = (int)a->M_out; p.N_out = (int)a->N_out; p.R_up = (int)a->R_up; p.R_down = (int)a->R_down;
     p.alpha = a->alpha;
-    for (int i = 0; i < 8; i++) p.lora_scales[i] = (a->lora_scales && i < (a->R_up + 15) / 16) ? a->lora_scales[i] : 1.0f;
+    for (int i = 0; i < MAX_RANK / 16; i++) p.lora_scales[i] = (a->lora_scales && i < (a->R_up + 15) / 16) ? a->lora_scales[i] : 1.0f;
     p.norm_q = (const uint16_t *)a->norm_q;
     p.norm_k = (const uint16_t *)a->norm_k;
     p.rotary = a->rotary_emb;
@@ -310,14 +321,14 @@ int gemm_int4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool no
     if (rc == SVDQ_OK && p.next_down) {
         // the column blocks' shares of the next layer's low-rank projection, added in ascending order
         const int quads = p.M_pad * p.R_down / 4;
-        hipLaunchKernelGGL(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
+        SVDQ_LAUNCH(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
                            p.next_lora_out, nblocks, p.M_pad, p.R_down);
         rc = check_launch("gemm_w4a4 (low-rank shares)");
     }
     if (rc == SVDQ_OK && p.vk) {
         // the row blocks' linear-attention sums, added per batch entry in ascending order of the rows
         const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * VK_HEAD_FLOATS;
-        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
+        SVDQ_LAUNCH(reduce_vk_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
                            p.vk_rows / g6::BM, heads);
         rc = check_launch("gemm_w4a4 (linear-attention sums)");
     }
@@ -347,7 +358,7 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     p.M_pad = (int)a->M_pad; p.N = (int)a->N; p.K = (int)a->K;
     p.M_out = (int)a->M_out; p.N_out = (int)a->N_out; p.R_up = (int)a->R_up;
     p.alpha = a->alpha;
-    for (int i = 0; i < 8; i++) p.lora_scales[i] = (a->lora_scales && i < (a->R_up + 15) / 16) ? a->lora_scales[i] : 1.0f;
+    for (int i = 0; i < MAX_RANK / 16; i++) p.lora_scales[i] = (a->lora_scales && i < (a->R_up + 15) / 16) ? a->lora_scales[i] : 1.0f;
     p.norm_q = (const uint16_t *)a->norm_q;
     p.norm_k = (const uint16_t *)a->norm_k;
     p.rotary = a->rotary_emb;
@@ -438,13 +449,13 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
     int rc = next ? launch_gemm_fp4_v5(p, nwg, st) : launch_gemm_fp4_v4(p, nwg, st);
     if (rc == SVDQ_OK && p.next_down) {
         const int quads = p.M_pad * p.R_down / 4;
-        hipLaunchKernelGGL(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
+        SVDQ_LAUNCH(reduce_shares_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, (const float4_t *)p.next_lora_part,
                            p.next_lora_out, p.N / 128, p.M_pad, p.R_down);
         rc = check_launch("gemm_w4a4 (low-rank shares)");
     }
     if (rc == SVDQ_OK && p.vk) {
         const int heads = p.N / 96, n = (p.M_pad / p.vk_rows) * heads * VK_HEAD_FLOATS;
-        hipLaunchKernelGGL(reduce_vk_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
+        SVDQ_LAUNCH(reduce_vk_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st, (const float *)p.vk_part, p.vk, p.M_pad / p.vk_rows,
                            p.vk_rows / 32, heads);
         rc = check_launch("gemm_w4a4 (linear-attention sums)");
     }
@@ -463,7 +474,7 @@ int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
     SVDQ_REQUIRE(a->K > 0 && a->K % 128 == 0, "gemm: K (%lld) must be a positive multiple of 128", (long long)a->K);
     SVDQ_REQUIRE(a->out || a->qout || a->out_q, "gemm: one of out / qout / out_q must be given");
     SVDQ_REQUIRE((a->lora_up != nullptr) == (a->lora_act_in != nullptr), "gemm: lora_up and lora_act_in go together");
-    SVDQ_REQUIRE(a->R_up >= 0 && a->R_up % 16 == 0 && a->R_up <= 128, "gemm: R_up (%lld) must be a multiple of 16, at most 128", (long long)a->R_up);
+    SVDQ_REQUIRE(a->R_up >= 0 && a->R_up % 16 == 0 && a->R_up <= MAX_RANK, "gemm: R_up (%lld) must be a multiple of 16, at most %d", (long long)a->R_up, MAX_RANK);
     SVDQ_REQUIRE((a->R_up > 0) == (a->lora_up != nullptr), "gemm: R_up and lora_up disagree");
     SVDQ_REQUIRE(a->k_split >= 0, "gemm: k_split must not be negative");
     if (a->out) {
@@ -498,7 +509,7 @@ int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
     }
     SVDQ_REQUIRE((a->next_lora_down != nullptr) == (a->next_lora_act_out != nullptr) && (a->next_lora_down != nullptr) == (a->R_down > 0),
                  "gemm: next_lora_down, next_lora_act_out and R_down go together");
-    SVDQ_REQUIRE(a->R_down >= 0 && a->R_down % 16 == 0 && a->R_down <= 128, "gemm: R_down (%lld) must be a multiple of 16, at most 128", (long long)a->R_down);
+    SVDQ_REQUIRE(a->R_down >= 0 && a->R_down % 16 == 0 && a->R_down <= MAX_RANK, "gemm: R_down (%lld) must be a multiple of 16, at most %d", (long long)a->R_down, MAX_RANK);
 
     if (a->rotary_emb) {
         SVDQ_REQUIRE(a->norm_q && a->norm_k, "gemm: rotary_emb needs norm_q and norm_k");
@@ -539,3 +550,24 @@ int gemm_entry(const svdq_gemm_args *a, void *stream, bool noalloc) {
 extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *a, void *stream) { return gemm_entry(a, stream, false); }
 
 extern "C" int svdq_gemm_w4a4_noalloc(const svdq_gemm_args *a, void *stream) { return gemm_entry(a, stream, true); }
+
+extern "C" int svdq_release_workspaces(void) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    int prev = 0;
+    if (hipGetDevice(&prev) != hipSuccess) return fail(SVDQ_ELAUNCH, "release_workspaces: cannot identify the current device");
+    int rc = SVDQ_OK;
+    auto release = [&](int dev, void *ptr) {
+        if (!ptr) return;
+        // everything enqueued on the block's device has finished before the block goes
+        if (hipSetDevice(dev) != hipSuccess || hipDeviceSynchronize() != hipSuccess || hipFree(ptr) != hipSuccess) {
+            (void)hipGetLastError();
+            rc = fail(SVDQ_ELAUNCH, "release_workspaces: cannot free a block on device %d", dev);
+        }
+    };
+    for (Workspace &w : g_ws) release(w.dev, w.ptr);
+    for (Retired &r : g_retired) release(r.dev, r.ptr);
+    g_ws.clear();
+    g_retired.clear();
+    (void)hipSetDevice(prev);
+    return rc;
+}

@@ -530,7 +530,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #pragma unroll
                 for (int k = 0; k < 2; k++) {
                     if (k == 1 && !two) break;
-                    const float ls = p.lora_scales[(s0 + k) < 8 ? (s0 + k) : 7];
+                    const float ls = p.lora_scales[s0 + k];
                     bf16x8_t la[4], lb[4], lb_rem[4];
 #pragma unroll
                     for (int t = 0; t < 4; t++) {
@@ -871,7 +871,7 @@ int launch_gemm_variant(const GemmParams &p, int nwg, hipStream_t stream) {
         if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
         lds_reserved[dev] = true;
     }
-    hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), LDS_BYTES, stream, p);
+    SVDQ_LAUNCH(kern, dim3(nwg), dim3(256), LDS_BYTES, stream, p);
     return check_launch("gemm_w4a4");
 }
 

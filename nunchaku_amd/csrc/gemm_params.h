@@ -7,6 +7,9 @@
 namespace svdq {
 
 
+// ranks of the low-rank branch: multiples of 16 up to this (the reference: MAX_RANK = 1024, lora.cuh:22)
+constexpr int MAX_RANK = 1024;
+
 constexpr int BM = 256, BN = 256;
 constexpr int STAGES = 4;
 // per stage: 8 KB A codes, 8 KB B codes, then 16 bytes of packed fp16 scale pairs per row / column:
@@ -174,7 +177,7 @@ struct GemmParams {
     int *counters;
     int M_pad, N, K, M_out, N_out, R_up, R_down;
     float alpha;
-    float lora_scales[8];
+    float lora_scales[MAX_RANK / 16];
     int gelu;
     int silu;  // x * sigmoid(x) before the store (next-layer variants only)
     // RMS norm + rotary embedding on the q and k heads of a fused QKV projection (next-layer variants only)
@@ -238,7 +241,7 @@ struct Params {
     int kparts;
     int M_pad, N, K, M_out, N_out, R_up, R_down;
     float alpha;
-    float lora_scales[8];
+    float lora_scales[MAX_RANK / 16];
     int gelu, silu;
     const uint16_t *norm_q, *norm_k;
     const float *rotary;

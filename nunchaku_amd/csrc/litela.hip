@@ -106,7 +106,7 @@ extern "C" int svdq_linearattn_vk_mul_q(void *q, const float *vk, int64_t batch,
     SVDQ_REQUIRE(num_tokens > 0 && num_tokens <= tokens_pad && tokens_pad < (1ll << 31), "vk_mul_q: num_tokens (%lld) must be in 1..tokens_pad (%lld)",
                  (long long)num_tokens, (long long)tokens_pad);
     SVDQ_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)vk % 16 == 0, "vk_mul_q: pointers must be 16-byte aligned");
-    hipLaunchKernelGGL(vk_mul_q_kernel, dim3((unsigned)((num_tokens + TOKENS_PER_WG - 1) / TOKENS_PER_WG), (unsigned)((heads + 3) / 4), (unsigned)batch), dim3(256), 0, (hipStream_t)stream,
+    SVDQ_LAUNCH(vk_mul_q_kernel, dim3((unsigned)((num_tokens + TOKENS_PER_WG - 1) / TOKENS_PER_WG), (unsigned)((heads + 3) / 4), (unsigned)batch), dim3(256), 0, (hipStream_t)stream,
                        (uint16_t *)q, vk, eps, (int)num_tokens, (int)tokens_pad, (int)heads);
     return check_launch("linearattn_vk_mul_q");
 }

@@ -36,6 +36,7 @@ struct QuantParams {
     float *lora_out;         // [M_pad, R]
     const float *smooth_rcp; // [K] or null
     int M, M_pad, K, R;
+    int rt_base;             // first 16-rank tile of the projection this launch computes (ranks above 128 take several launches)
 };
 
 constexpr uint32_t RSRC_WORD3 = 0x00020000;  // raw buffer, 32-bit data format
@@ -54,7 +55,11 @@ constexpr uint32_t RSRC_WORD3 = 0x00020000;  // raw buffer, 32-bit data format
 // chunk, one chunk ahead, into an LDS double buffer; with chunks split among the waves every wave fetched its own
 // chunks' operands from the L2, one dependent request after the other.  No sums cross waves, so there is no
 // reduction at the end either.
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS>
+//
+// Ranks above 16 RT_MAX: a launch projects onto the rank tiles [rt_base, rt_base + RT_MAX) only (its accumulators
+// live in registers), so the operator launches the kernel once per window of 128 ranks; the launches after the
+// first (QUANT false) read x again, which the caches still hold, and neither quantize nor store codes.
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS, bool QUANT = true>
 __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams p) {
     // smoothing factors [K] during the walk; then, chunks split: [NW waves][MT][RT][64][4] partial projections;
     // rows split: behind the factors two buffers of [4 steps][RT][64 lanes] x 16 bytes of proj_down
@@ -64,7 +69,8 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
     const int r = lane & 15, q = lane >> 4;
     const int row0 = ROWS ? (blockIdx.x * NW + wave) * (16 * MT) : blockIdx.x * (16 * MT);
     const int kgroups = p.K / 64;
-    const int RT = p.R / 16;
+    const int RT_all = p.R / 16;                                                         // rank tiles of proj_down and lora_out
+    const int RT = RT_all - p.rt_base < RT_MAX ? RT_all - p.rt_base : RT_MAX;            // rank tiles of this launch
     const int nchunks = p.K / 128;
 
     float4_t acc[MT][RT_MAX];
@@ -112,7 +118,7 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
     // proj_down as a buffer too: empty when there is no low-rank branch, so that its requests need no branch
     const __amdgpu_buffer_rsrc_t drsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.down, 0, RT > 0 ? p.K * p.R * 2 : 0, RSRC_WORD3);
     auto load_down = [&](int c, int i, int rt) {
-        return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(drsrc, lane * 16, (((c * 4 + i) * RT + (rt < RT ? rt : 0)) * 64) * 16, 0));
+        return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(drsrc, lane * 16, (((c * 4 + i) * RT_all + p.rt_base + (rt < RT ? rt : 0)) * 64) * 16, 0));
     };
 
     // DEPTH chunks are requested ahead of the one being worked on
@@ -122,7 +128,7 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
 #pragma unroll
     for (int s = 0; s < DEPTH; s++) load_x(cfirst + s * CSTEP, xv[s]);
 
-    if (SMOOTH == 1) {
+    if (QUANT && SMOOTH == 1) {
         for (int k = threadIdx.x * 4; k < p.K; k += 64 * NW * 4) *(float4_t *)&lds[k] = *(const float4_t *)(p.smooth_rcp + k);
         __syncthreads();
     }
@@ -213,7 +219,7 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
 
         // ---- smooth, quantize, store
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
+        for (int mt = 0; mt < (QUANT ? MT : 0); mt++) {
             const int row = row0 + 16 * mt + r;
             float y[32];
 #pragma unroll
@@ -314,45 +320,47 @@ walked:
             for (int rt = 0; rt < RT_MAX; rt++)
                 if (rt < RT) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) p.lora_out[(size_t)(row0 + 16 * mt + 4 * q + i) * p.R + 16 * rt + r] = acc[mt][rt][i];
+                    for (int i = 0; i < 4; i++) p.lora_out[(size_t)(row0 + 16 * mt + 4 * q + i) * p.R + 16 * (p.rt_base + rt) + r] = acc[mt][rt][i];
                 }
         return;
     }
     // ---- reduce the waves' partial projections and write lora_act[row][rank]
     if (RT > 0) {
-        if (SMOOTH == 1) __syncthreads();  // the factors in LDS are not needed any more
+        if (QUANT && SMOOTH == 1) __syncthreads();  // the factors in LDS are not needed any more
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int rt = 0; rt < RT_MAX; rt++)
                 if (rt < RT) *(float4_t *)&lds[(((wave * MT + mt) * RT + rt) * 64 + lane) * 4] = acc[mt][rt];
         __syncthreads();
-        const int total = 16 * MT * p.R;
+        const int RW = 16 * RT;  // ranks of this launch
+        const int total = 16 * MT * RW;
         for (int idx = threadIdx.x; idx < total; idx += 64 * NW) {
-            const int row = idx / p.R, rank = idx % p.R;
+            const int row = idx / RW, rank = idx % RW;
             const int mt = row / 16, rr = row % 16, rt = rank / 16, rc = rank % 16;
             const int src_lane = 16 * (rr / 4) + rc, i = rr % 4;  // 16x16 MFMA result layout
             float sum = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; w++) sum += lds[(((w * MT + mt) * RT + rt) * 64 + src_lane) * 4 + i];
-            p.lora_out[(size_t)(row0 + row) * p.R + rank] = sum;
+            p.lora_out[(size_t)(row0 + row) * p.R + 16 * p.rt_base + rank] = sum;
         }
     }
 }
 
 constexpr size_t SMOOTH_LDS_MAX = 64 * 1024;  // two workgroups of a compute unit must fit side by side
 
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS = false>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS = false, bool QUANT = true>
 int launch_as(const QuantParams &p, hipStream_t stream) {
-    size_t smem = (size_t)NW * MT * (p.R / 16) * 64 * 4 * sizeof(float);
+    const int rt_launch = p.R / 16 - p.rt_base < RT_MAX ? p.R / 16 - p.rt_base : RT_MAX;
+    size_t smem = (size_t)NW * MT * rt_launch * 64 * 4 * sizeof(float);
     if (SMOOTH == 1 && (size_t)p.K * 4 > smem) smem = (size_t)p.K * 4;
     if (ROWS) smem = (SMOOTH == 1 ? (size_t)p.K * 4 : 0) + 2 * (size_t)(p.R / 16) * 4096;
-    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH, GLU, ROWS>;
+    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH, GLU, ROWS, QUANT>;
     if (smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "quantize: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(kern, dim3(p.M_pad / (16 * MT * (ROWS ? NW : 1))), dim3(64 * NW), smem, stream, p);
+    SVDQ_LAUNCH(kern, dim3(p.M_pad / (16 * MT * (ROWS ? NW : 1))), dim3(64 * NW), smem, stream, p);
     return check_launch("quantize_w4a4_act_fuse_lora");
 }
 
@@ -361,6 +369,17 @@ int launch(const QuantParams &p, hipStream_t stream) {
     if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0, GLU, ROWS>(p, stream);
     if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1, GLU, ROWS>(p, stream);
     return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2, GLU, ROWS>(p, stream);
+}
+
+// the rank tiles from 8 on, 8 per launch: projection only (no smoothing factors, no codes, either precision)
+template <int NW, int MT, bool GLU>
+int project_further(const QuantParams &p0, hipStream_t stream) {
+    QuantParams p = p0;
+    for (p.rt_base = 8; p.rt_base < p.R / 16; p.rt_base += 8) {
+        const int rc = launch_as<NW, MT, 8, 1, false, 0, GLU, false, false>(p, stream);
+        if (rc != SVDQ_OK) return rc;
+    }
+    return SVDQ_OK;
 }
 
 template <bool FP4, bool GLU>
@@ -374,11 +393,13 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         if (RT <= 2) return launch<4, 1, 2, 1, FP4, true>(p, stream);
         if (RT <= 4) return launch<4, 1, 4, 1, FP4, true>(p, stream);
         if (RT <= 8) return launch<4, 1, 8, 1, FP4, true>(p, stream);
+        const int rc = launch<4, 1, 8, 1, FP4, true>(p, stream);
+        return rc != SVDQ_OK ? rc : project_further<4, 1, true>(p, stream);
     } else {
         // High ranks with enough rows to give every compute unit work: the waves split the rows and share each
         // chunk of proj_down through LDS (M = 18432, K = 3072: rank 128 68 us against 122, rank 64 51 against 71;
         // at M = 4608 the few large workgroups lose: 65 against 42).
-        if (RT > 4 && p.M_pad >= 128 * 128) return launch<4, 2, 8, 1, FP4, false, true>(p, stream);
+        if (RT > 4 && RT <= 8 && p.M_pad >= 128 * 128) return launch<4, 2, 8, 1, FP4, false, true>(p, stream);
         if (RT > 2 && RT <= 4 && p.M_pad >= 256 * 64) return launch<4, 1, 4, 1, FP4, false, true>(p, stream);
         // Up to one 16-row workgroup per compute unit (256 of them) the walk over K is what takes the time: eight waves
         // split it (M = 256 ... 4096 at K = 3072: 7.9 ... 10.1 us against 9.0 ... 11.3 with four; K = 12288, M = 256:
@@ -387,8 +408,10 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         if (RT <= 2) return p.M_pad >= 8192 ? launch<4, 2, 2, 1, FP4, false>(p, stream) : launch<4, 1, 2, 1, FP4, false>(p, stream);
         if (RT <= 4) return launch<4, 2, 4, 1, FP4, false>(p, stream);
         if (RT <= 8) return launch<4, 2, 8, 1, FP4, false>(p, stream);
+        // ranks above 128: the first 128 with the codes, the rest in further launches over the same rows
+        const int rc = launch<4, 2, 8, 1, FP4, false>(p, stream);
+        return rc != SVDQ_OK ? rc : project_further<4, 2, false>(p, stream);
     }
-    return fail(SVDQ_EUNSUPPORTED, "quantize: rank %d > 128 is not supported", p.R);
 }
 
 }  // namespace
@@ -399,7 +422,7 @@ extern "C" int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *a, voi
     SVDQ_REQUIRE(a->M > 0 && a->M_pad >= a->M && a->M_pad % 256 == 0, "quantize: M_pad (%lld) must be a multiple of 256 and >= M (%lld)",
                  (long long)a->M_pad, (long long)a->M);
     SVDQ_REQUIRE(a->K > 0 && a->K % 128 == 0, "quantize: K (%lld) must be a multiple of 128", (long long)a->K);
-    SVDQ_REQUIRE(a->R >= 0 && a->R % 16 == 0, "quantize: rank (%lld) must be a multiple of 16", (long long)a->R);
+    SVDQ_REQUIRE(a->R >= 0 && a->R % 16 == 0 && a->R <= 1024, "quantize: rank (%lld) must be a multiple of 16, at most 1024 (lora.cuh:22)", (long long)a->R);
     SVDQ_REQUIRE(a->R == 0 || (a->lora_down && a->lora_act_out), "quantize: lora_down/lora_act_out must be given when R > 0");
     SVDQ_REQUIRE(a->M_pad < (1ll << 31) / 4 && a->K < (1 << 24) && a->K * a->R < (1ll << 30), "quantize: shape too large");
     SVDQ_REQUIRE(((uintptr_t)a->input % 16 == 0) && ((uintptr_t)a->output % 16 == 0) && ((uintptr_t)a->lora_down % 16 == 0) &&
@@ -413,6 +436,7 @@ extern "C" int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *a, voi
     p.lora_out = a->lora_act_out;
     p.smooth_rcp = a->smooth_rcp;
     p.M = (int)a->M; p.M_pad = (int)a->M_pad; p.K = (int)a->K; p.R = (int)a->R;
+    p.rt_base = 0;
     hipStream_t s = (hipStream_t)stream;
     if (a->fuse_glu) return a->fp4 ? dispatch<true, true>(p, s) : dispatch<false, true>(p, s);
     return a->fp4 ? dispatch<true, false>(p, s) : dispatch<false, false>(p, s);

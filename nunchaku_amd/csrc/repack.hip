@@ -222,14 +222,14 @@ int svdq_repack_qweight(const void *src, void *dst, int64_t N, int64_t K, int fp
     if (!fp4) {
         const int64_t slots = ((N + WGT_BLOCK_COLS - 1) / WGT_BLOCK_COLS) * (K / 64) * 8 * 64;
         SVDQ_REQUIRE((uintptr_t)dst % 16 == 0, "repack_qweight: dst must be 16-byte aligned");
-        hipLaunchKernelGGL(repack_qweight_e2m3_kernel, dim3(blocks_for(slots)), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
+        SVDQ_LAUNCH(repack_qweight_e2m3_kernel, dim3(blocks_for(slots)), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
                            (uint8_t *)dst, N, K);
         return check_launch("repack_qweight");
     }
     const int64_t total = N * K / 8;
     unsigned grid = blocks_for(total);
     if (grid > 65536u) grid = 65536u;
-    hipLaunchKernelGGL(repack_qweight_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
+    SVDQ_LAUNCH(repack_qweight_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
                        (uint32_t *)dst, N, K);
     return check_launch("repack_qweight");
 }
@@ -239,7 +239,7 @@ int svdq_repack_wscales(const void *src, void *dst_scales, int64_t N, int64_t K,
     SVDQ_REQUIRE(N > 0 && K > 0 && N % 128 == 0 && K % 64 == 0, "repack_wscales: N %% 128 and K %% 64 must be 0");
     SVDQ_REQUIRE((uintptr_t)dst_scales % 16 == 0, "repack_wscales: dst must be 16-byte aligned");
     const int64_t total = ((N + WGT_BLOCK_COLS - 1) / WGT_BLOCK_COLS) * (K / 64) * WGT_BLOCK_COLS;
-    hipLaunchKernelGGL(repack_wscales_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
+    SVDQ_LAUNCH(repack_wscales_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
                        (unsigned long long *)dst_scales, N, K / 64);
     return check_launch("repack_wscales");
 }
@@ -247,7 +247,7 @@ int svdq_repack_wscales(const void *src, void *dst_scales, int64_t N, int64_t K,
 int svdq_repack_wmscales(const void *src, void *dst_scales, void *dst_colnorm, int64_t N, int64_t K, void *stream) {
     SVDQ_REQUIRE(src && dst_scales && dst_colnorm, "repack_wmscales: null pointer");
     SVDQ_REQUIRE(N > 0 && K > 0 && N % 128 == 0 && K % 64 == 0, "repack_wmscales: N %% 128 and K %% 64 must be 0");
-    hipLaunchKernelGGL(repack_wmscales_kernel, dim3(blocks_for(N)), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)src,
+    SVDQ_LAUNCH(repack_wmscales_kernel, dim3(blocks_for(N)), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)src,
                        (_Float16 *)dst_scales, (float *)dst_colnorm, N, K / 16);
     return check_launch("repack_wmscales");
 }
@@ -255,7 +255,7 @@ int svdq_repack_wmscales(const void *src, void *dst_scales, void *dst_colnorm, i
 int svdq_repack_vector(const void *src, void *dst, int64_t N, void *stream) {
     SVDQ_REQUIRE(src && dst && src != dst, "repack_vector: null or aliased pointer");
     SVDQ_REQUIRE(N > 0 && N % 128 == 0, "repack_vector: N (%lld) must be a multiple of 128", (long long)N);
-    hipLaunchKernelGGL(repack_vector_kernel, dim3(blocks_for(N)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
+    SVDQ_LAUNCH(repack_vector_kernel, dim3(blocks_for(N)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
                        (uint16_t *)dst, N);
     return check_launch("repack_vector");
 }
@@ -263,7 +263,7 @@ int svdq_repack_vector(const void *src, void *dst, int64_t N, void *stream) {
 int svdq_repack_smooth(const void *src, void *dst_rcp, int64_t K, void *stream) {
     SVDQ_REQUIRE(src && dst_rcp, "repack_smooth: null pointer");
     SVDQ_REQUIRE(K > 0 && K % 128 == 0, "repack_smooth: K (%lld) must be a multiple of 128", (long long)K);
-    hipLaunchKernelGGL(repack_smooth_kernel, dim3(blocks_for(K)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
+    SVDQ_LAUNCH(repack_smooth_kernel, dim3(blocks_for(K)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
                        (float *)dst_rcp, K);
     return check_launch("repack_smooth");
 }
@@ -271,7 +271,7 @@ int svdq_repack_smooth(const void *src, void *dst_rcp, int64_t K, void *stream) 
 int svdq_repack_lora_down(const void *src, void *dst, int64_t K, int64_t R, void *stream) {
     SVDQ_REQUIRE(src && dst && src != dst, "repack_lora_down: null or aliased pointer");
     SVDQ_REQUIRE(K > 0 && K % 128 == 0 && R > 0 && R % 16 == 0, "repack_lora_down: K %% 128 and R %% 16 must be 0");
-    hipLaunchKernelGGL(repack_lora_down_kernel, dim3(blocks_for(K * R)), dim3(256), 0, (hipStream_t)stream,
+    SVDQ_LAUNCH(repack_lora_down_kernel, dim3(blocks_for(K * R)), dim3(256), 0, (hipStream_t)stream,
                        (const uint16_t *)src, (uint16_t *)dst, K, R);
     return check_launch("repack_lora_down");
 }
@@ -279,7 +279,7 @@ int svdq_repack_lora_down(const void *src, void *dst, int64_t K, int64_t R, void
 int svdq_repack_lora_up(const void *src, void *dst, int64_t N, int64_t R, void *stream) {
     SVDQ_REQUIRE(src && dst && src != dst, "repack_lora_up: null or aliased pointer");
     SVDQ_REQUIRE(N > 0 && N % 16 == 0 && R > 0 && R % 16 == 0, "repack_lora_up: N %% 16 and R %% 16 must be 0");
-    hipLaunchKernelGGL(repack_lora_up_kernel, dim3(blocks_for(N * R)), dim3(256), 0, (hipStream_t)stream,
+    SVDQ_LAUNCH(repack_lora_up_kernel, dim3(blocks_for(N * R)), dim3(256), 0, (hipStream_t)stream,
                        (const uint16_t *)src, (uint16_t *)dst, N, R);
     return check_launch("repack_lora_up");
 }
@@ -287,7 +287,7 @@ int svdq_repack_lora_up(const void *src, void *dst, int64_t N, int64_t R, void *
 int svdq_repack_rotemb(const void *src, void *dst, int64_t rows, void *stream) {
     SVDQ_REQUIRE(src && dst && src != dst, "repack_rotemb: null or aliased pointer");
     SVDQ_REQUIRE(rows > 0 && rows % 32 == 0, "repack_rotemb: rows (%lld) must be a positive multiple of 32", (long long)rows);
-    hipLaunchKernelGGL(repack_rotemb_kernel, dim3(blocks_for(rows * 128)), dim3(256), 0, (hipStream_t)stream, (const float *)src,
+    SVDQ_LAUNCH(repack_rotemb_kernel, dim3(blocks_for(rows * 128)), dim3(256), 0, (hipStream_t)stream, (const float *)src,
                        (float *)dst, rows);
     return check_launch("repack_rotemb");
 }

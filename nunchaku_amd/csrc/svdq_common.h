@@ -22,9 +22,17 @@ inline int fail(int code, const char *fmt, ...) {
     va_end(ap);
     return code;
 }
+// A launch is reported by what hipGetLastError() says right after it.  That call returns the last error of the
+// thread, whoever caused it, so an error left behind by an earlier call (this library's or anybody else's) is
+// discarded first: what check_launch reports then belongs to the launch it follows.
+#define SVDQ_LAUNCH(...)                 \
+    do {                                 \
+        (void)hipGetLastError();         \
+        hipLaunchKernelGGL(__VA_ARGS__); \
+    } while (0)
 inline int check_launch(const char *what) {
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+    if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "%s: %s (%s)", what, hipGetErrorString(e), hipGetErrorName(e));
     return SVDQ_OK;
 }
 #define SVDQ_REQUIRE(cond, ...) \

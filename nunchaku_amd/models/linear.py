@@ -191,8 +191,8 @@ class SVDQW4A4Linear(nn.Module):
         src/Linear.cpp:124-134)."""
         if proj_down.shape[0] != self.in_features or proj_up.shape[0] != self.out_features or proj_down.shape[1] != proj_up.shape[1]:
             raise ValueError(f"expected proj_down [{self.in_features}, R] and proj_up [{self.out_features}, R], got {tuple(proj_down.shape)} and {tuple(proj_up.shape)}")
-        if proj_down.shape[1] % 16 != 0 or proj_down.shape[1] > 128:
-            raise ValueError("the rank must be a multiple of 16, at most 128")
+        if proj_down.shape[1] % 16 != 0 or proj_down.shape[1] > 1024:
+            raise ValueError("the rank must be a multiple of 16, at most 1024 (the reference's MAX_RANK, lora.cuh:22)")
         dev, dt = self.proj_down.device, self.proj_down.dtype
         self.proj_down = nn.Parameter(proj_down.detach().to(device=dev, dtype=dt).contiguous(), requires_grad=False)
         self.proj_up = nn.Parameter(proj_up.detach().to(device=dev, dtype=dt).contiguous(), requires_grad=False)

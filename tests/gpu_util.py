@@ -44,3 +44,26 @@ def make_oracle(layer: synth.LogicalLayer, act_unsigned=False):
         layer.wq, layer.ws, layer.smooth, layer.proj_down, layer.proj_up, layer.bias,
         fp4=layer.fp4, wtscale=layer.wtscale, wcscales=layer.wcscales, act_unsigned=act_unsigned,
     )
+
+
+class Guarded:
+    """A tensor placed inside a larger buffer filled with a byte pattern: ``check()`` asserts that the bands before and
+    behind it still hold the pattern, i.e. that no kernel wrote outside the tensor."""
+
+    PATTERN = 0xA5
+
+    def __init__(self, shape, dtype, dev, band: int = 1 << 16):
+        n = 1
+        for d in shape:
+            n *= d
+        self.nbytes = n * torch.empty((), dtype=dtype).element_size()
+        self.band = band
+        padded = (self.nbytes + 255) // 256 * 256
+        self.raw = torch.full((band + padded + band,), self.PATTERN, dtype=torch.uint8, device=dev)
+        self.t = self.raw[band:band + self.nbytes].view(dtype).view(*shape)
+
+    def check(self, name: str) -> None:
+        before = self.raw[:self.band]
+        behind = self.raw[self.band + self.nbytes:]
+        assert bool((before == self.PATTERN).all()), f"{name}: bytes in front of the tensor were overwritten"
+        assert bool((behind == self.PATTERN).all()), f"{name}: bytes behind the tensor were overwritten"

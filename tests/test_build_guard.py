@@ -1,0 +1,141 @@
+"""What the hot kernels' performance and correctness rest on in the compiler's output, checked on the CPU (hipcc
+cross-compiles gfx950 without a GPU).
+
+* Registers.  ``g6::gemm6_kernel`` holds 128 accumulators per lane and runs two workgroups per compute unit: it must
+  fit 256 vector registers without scratch.  A compiler that spills there costs time silently (spills of 236 and 518
+  registers were seen while the kernel was written).  The NVFP4 kernel's figures are recorded with a ceiling.
+* Flags across inline assembly.  The asynchronous global -> LDS copies are inline assembly that writes ``m0`` and, where
+  it adds, the scalar condition code (SCC).  A build whose asm statements did not declare that had the compiler keep the
+  carry of a 64-bit pointer addition (``s_add_u32`` ... ``s_addc_u32``) and the result of ``ng < 2`` in SCC across such
+  a statement: the carry was lost whenever an operand tensor straddled a 4 GiB address boundary, and the kernel then
+  read 4 GiB below its operands (a GPU memory fault that depended on where the allocator had placed the tensors).  The
+  generated code is scanned: after an asm statement that writes SCC, nothing may read SCC before something else has
+  written it.
+"""
+
+import re
+import subprocess
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+import pytest
+
+from nunchaku_amd import _native as nv
+
+CSRC = Path(nv.__file__).resolve().parent / "csrc"
+
+SCC_READERS = re.compile(r"^\s*(s_cbranch_scc[01]|s_cselect_b(32|64)|s_addc_u32|s_subb_u32|s_cmov_b(32|64))\b")
+SCC_WRITERS = re.compile(
+    r"^\s*(s_cmp_|s_cmpk_|s_add_[ui]32|s_sub_[ui]32|s_addk_|s_mulk_|s_and_|s_or_|s_xor_|s_andn2_|s_orn2_|s_nand_|s_nor_|s_xnor_|"
+    r"s_lshl_b|s_lshr_b|s_ashr_i|s_bfe_|s_min_|s_max_|s_abs_|s_absdiff_|s_bitcmp|s_not_|s_wqm_|s_quadmask_|s_lshl[1-4]_add_|s_bcnt|"
+    r"s_ff[01]_|s_flbit_)")
+CONTROL = re.compile(r"^\s*(s_branch|s_cbranch_|s_endpgm|s_setpc_|s_swappc_)")
+
+
+def compile_variant(src: str, variant: int, tmp: str):
+    out = Path(tmp) / f"{src}_{variant}.s"
+    flags = [f for f in nv.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    res = subprocess.run(["/opt/rocm/bin/hipcc", *flags, f"-DSVDQ_VARIANT={variant}", "-S", "--cuda-device-only",
+                          "-Rpass-analysis=kernel-resource-usage", str(CSRC / src), "-o", str(out)], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-3000:]
+    usage = {}
+    name = None
+    for line in res.stderr.splitlines():
+        m = re.search(r"remark: .*Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            usage[name] = {}
+        m = re.search(r"remark: .*?\s+([A-Za-z ]+?)(?: \[[^\]]*\])?: (\d+)", line)
+        if m and name and "Function Name" not in line:
+            usage[name][m.group(1).strip()] = int(m.group(2))
+    return usage, out.read_text().splitlines()
+
+
+def scc_live_across_asm(lines):
+    """(line number, text) of every SCC reader that follows an SCC-writing inline-asm statement with no SCC writer
+    between them, in straight-line order; control flow or a label right behind such a statement is reported too (the
+    compiler treats a declared clobber as a definition, so neither occurs in a correct build)."""
+    bad = []
+    i = 0
+    while i < len(lines):
+        if "#ASMSTART" in lines[i]:
+            j = i
+            while "#ASMEND" not in lines[j]:
+                j += 1
+            if any(SCC_WRITERS.match(b) for b in lines[i + 1:j]):
+                k = j + 1
+                while k < len(lines):
+                    s = lines[k]
+                    if SCC_READERS.match(s):
+                        bad.append((k + 1, s.strip()))
+                        break
+                    if SCC_WRITERS.match(s) or "#ASMSTART" in s or CONTROL.match(s) or re.match(r"^\.LBB\d+_\d+:", s.strip()):
+                        break
+                    k += 1
+            i = j
+        i += 1
+    return bad
+
+
+def test_scanner_finds_a_carry_kept_across_an_asm_add():
+    bad = """
+	s_add_u32 s26, s8, 0x1800
+	;;#ASMSTART
+	s_add_u32 m0, s44, s11
+	s_nop 0
+	global_load_lds_dwordx4 v1, s[6:7] offset:1024
+	;;#ASMEND
+	s_addc_u32 s27, s9, 0
+""".splitlines()
+    assert scc_live_across_asm(bad) == [(8, "s_addc_u32 s27, s9, 0")]
+    good = """
+	;;#ASMSTART
+	s_add_u32 m0, s44, s11
+	;;#ASMEND
+	s_add_u32 s26, s8, 0x1800
+	s_addc_u32 s27, s9, 0
+""".splitlines()
+    assert scc_live_across_asm(good) == []
+
+
+@pytest.fixture(scope="module")
+def compiled():
+    units = [("gemm6_variant.hip", 0), ("gemm6_variant.hip", 1), ("gemm_variant.hip", 4), ("gemm_variant.hip", 5)]
+    with tempfile.TemporaryDirectory(prefix="svdq_guard_") as tmp:
+        with ThreadPoolExecutor(max_workers=4) as pool:
+            results = list(pool.map(lambda u: compile_variant(u[0], u[1], tmp), units))
+    return dict(zip(units, results))
+
+
+def kernel_usage(usage, fragment):
+    hits = [v for k, v in usage.items() if fragment in k]
+    assert len(hits) == 1, list(usage)
+    return hits[0]
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_int4_gemm_fits_its_registers(compiled, variant):
+    usage, _ = compiled[("gemm6_variant.hip", variant)]
+    u = kernel_usage(usage, "gemm6_kernel")
+    print(u)
+    assert u["VGPRs"] <= 256 and u["AGPRs"] == 0, u
+    assert u["ScratchSize"] == 0, f"gemm6_kernel spills: {u}"
+    assert u["Occupancy"] >= 2, u
+
+
+@pytest.mark.parametrize("variant,max_scratch", [(4, 128), (5, 256)])
+def test_nvfp4_gemm_register_figures(compiled, variant, max_scratch):
+    usage, _ = compiled[("gemm_variant.hip", variant)]
+    u = kernel_usage(usage, "gemm_w4a4_kernel")
+    print(u)
+    assert u["VGPRs"] + u["AGPRs"] <= 512, u
+    # the epilogue keeps some values in scratch; the main loop must not (a much larger figure means it does)
+    assert u["ScratchSize"] <= max_scratch, u
+
+
+@pytest.mark.parametrize("unit", [("gemm6_variant.hip", 0), ("gemm6_variant.hip", 1), ("gemm_variant.hip", 4), ("gemm_variant.hip", 5)])
+def test_no_condition_code_kept_across_inline_asm(compiled, unit):
+    _, lines = compiled[unit]
+    assert sum("#ASMSTART" in l for l in lines) > 0
+    assert scc_live_across_asm(lines) == []

@@ -86,9 +86,9 @@ def test_quantize_rejects_bad_arguments(lib):
     assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
     assert b"aligned" in lib.svdq_last_error()
     a.input = 16
-    a.R = 144
+    a.R = 1040  # the reference's MAX_RANK is 1024 (lora.cuh:22)
     a.fuse_glu = 1
-    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -2
+    assert lib.svdq_quantize_w4a4_act_fuse_lora(ctypes.byref(a), None) == -1
     assert b"rank" in lib.svdq_last_error()
 
 

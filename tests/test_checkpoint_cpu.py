@@ -73,6 +73,12 @@ def test_lora_scales_per_16_ranks():
         m.update_lora(torch.zeros(128, 24, dtype=torch.bfloat16), torch.zeros(128, 24, dtype=torch.bfloat16))
     with pytest.raises(ValueError):
         m.update_lora(torch.zeros(64, 32, dtype=torch.bfloat16), torch.zeros(128, 32, dtype=torch.bfloat16))
+    # the rank grows with what is loaded (src/Linear.cpp:124-134): a rank-128 LoRA behind the layer's own 32 ranks
+    m.update_lora(torch.zeros(128, 160, dtype=torch.bfloat16), torch.zeros(128, 160, dtype=torch.bfloat16))
+    m.set_lora_scale(32, 0.5)
+    assert m.rank == 160 and m.lora_scales == [1.0, 1.0] + [0.5] * 8
+    with pytest.raises(ValueError):  # the reference's MAX_RANK (lora.cuh:22)
+        m.update_lora(torch.zeros(128, 1040, dtype=torch.bfloat16), torch.zeros(128, 1040, dtype=torch.bfloat16))
 
 
 def test_safetensors_round_trip(tmp_path):

@@ -69,11 +69,12 @@ def test_load_toy_checkpoint_and_run_every_layer(dev, tmp_path, fp4_blocks):
         assert rel <= 2e-2, rel
 
 
-def test_lora_hot_swap_rank_growth_and_scales(dev):
+@pytest.mark.parametrize("R2", [16, 128, 224])  # a rank-128 user LoRA behind a stock rank-32 branch is rank 160
+def test_lora_hot_swap_rank_growth_and_scales(dev, R2):
     from nunchaku_amd import checkpoint
     from nunchaku_amd.models.linear import SVDQW4A4Linear
 
-    N, K, R, R2, M = 256, 256, 32, 16, 300
+    N, K, R, M = 256, 256, 32, 300
     announce(f"lora hot swap N={N} K={K} rank {R} + {R2}")
     layer = synth.make_layer(N, K, R, seed=21)
     mod = SVDQW4A4Linear(K, N, rank=R, device=dev)
@@ -103,7 +104,7 @@ def test_lora_hot_swap_rank_growth_and_scales(dev):
         from oracle import quant
 
         want = olin.gemm_w4a4(quant.dequant_int4(codes, scales), ref.w_deq, bias=ref.bias, lora_act_in=lora, lora_up=ref.proj_up,
-                              lora_scales=[1.0, 1.0, strength])[:M]
+                              lora_scales=[1.0, 1.0] + [strength] * (R2 // 16))[:M]
         check_output(y, want)
         if strength == 0.0:
             assert torch.equal(y, y0)  # the appended ranks switched off: the original layer, bit for bit

@@ -1,7 +1,8 @@
 """A seeded sweep over shapes and epilogue options of the two operators against the oracle: ragged token counts, N that is
-not a multiple of the INT4 kernel's 256-column tile, every rank from 0 to 128, with and without bias, per-channel scales,
-alpha, low-rank scale factors, tiles split along K, both precisions.  Every case is small enough for the CPU oracle to
-check every element."""
+not a multiple of the INT4 kernel's 256-column tile, ranks from 0 to 128 and a few up to 1024 (the reference's limit,
+lora.cuh:22), with and without bias, per-channel scales, alpha, low-rank scale factors, tiles split along K, both
+precisions.  Every case is small enough for the CPU oracle to check every element.  Every buffer the two operators write
+lies between bands of a byte pattern, which must be intact afterwards."""
 
 import random
 
@@ -10,7 +11,7 @@ import pytest
 import torch
 
 from conftest import announce
-from gpu_util import check_output, make_module, make_oracle
+from gpu_util import Guarded, check_output, make_module, make_oracle
 from oracle import layouts as L
 from oracle import synth
 
@@ -41,6 +42,17 @@ def _cases():
         opts = dict(bias=rng.random() < 0.7, scales=rng.random() < 0.4, alpha=rng.choice([1.0, 0.5]) if not fp4 else None,
                     lora_scales=rng.random() < 0.4, k_split=None)
         cases.append((i, M, K, N, R, fp4, opts))
+    # ranks above 128 (a stock rank-32 branch with a rank-128 user LoRA appended is 160): the quantize operator
+    # projects in windows of 128 ranks, the GEMM's up projection walks all of them
+    rng = random.Random(99)
+    for i, R in zip(range(200, 208), [160, 256, 160, 272, 1024, 256, 144, 512]):
+        fp4 = i % 4 == 3
+        M = rng.choice([100, 256, 300, 640])
+        K = 128 * rng.randint(1, 6)
+        N = 128 * rng.randint(1, 6)
+        opts = dict(bias=rng.random() < 0.7, scales=rng.random() < 0.4, alpha=rng.choice([1.0, 0.5]) if not fp4 else None,
+                    lora_scales=i % 2 == 0, k_split=None)
+        cases.append((i, M, K, N, R, fp4, opts))
     return cases
 
 
@@ -65,9 +77,20 @@ def test_layer_sweep(dev, i, M, K, N, R, fp4, opts, monkeypatch):
     lora_scales = None
     if opts["lora_scales"] and R:
         lora_scales = [float(v) for v in (0.25 + 1.5 * torch.rand((R + 15) // 16, generator=g)).tolist()]
-    qx, asc, la = m.quantize(x.to(dev))
+    from nunchaku_amd import packing
+    from nunchaku_amd.ops import svdq_quantize_w4a4_act_fuse_lora
+
     t = m.native_tensors()
-    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    M_pad = (M + 255) // 256 * 256
+    G = 16 if fp4 else 64
+    g_qx = Guarded((M_pad, packing.act_nbytes_per_row(K, fp4)), torch.uint8, dev)
+    g_asc = Guarded((K // G, M_pad), torch.float8_e4m3fn if fp4 else torch.bfloat16, dev)
+    g_la = Guarded((M_pad, R), torch.float32, dev)
+    g_out = Guarded((M, N), torch.bfloat16, dev)
+    qx, asc, la = svdq_quantize_w4a4_act_fuse_lora(x.to(dev), output=g_qx.t, oscales=g_asc.t, lora_down=t["proj_down"],
+                                                   lora_act_out=g_la.t, smooth=t["smooth_factor"], fp4=fp4)
+    out = g_out.t
+    out.fill_(float("nan"))
     monkeypatch.setattr(gemm_mod, "K_SPLIT", opts["k_split"])
     wcs = None
     if fp4:
@@ -82,6 +105,8 @@ def test_layer_sweep(dev, i, M, K, N, R, fp4, opts, monkeypatch):
         kw.update(lora_act_in=la, lora_up=t["proj_up"])
     svdq_gemm_w4a4(**kw)
     torch.cuda.synchronize()
+    for name, gd in (("quantized activations", g_qx), ("activation scales", g_asc), ("lora_act", g_la), ("out", g_out)):
+        gd.check(name)
     assert not torch.isnan(out.float()).any()
     codes, scales, lora = ref.quantize(x)
     from oracle import linear as olin
