@@ -18,8 +18,8 @@
  * Notation: M tokens, M_pad = M rounded up to 256, K in-features, N out-features, R low-rank rank,
  * G group size (64 for INT4, 16 for NVFP4).
  *
- * INT4 operands (activations and weights alike) are held as E2M3 (fp6) patterns of code / 2 -- exact
- * for every code in [-8, 15] -- in "fragments": one operand of the fp6 matrix instruction, 32 rows x
+ * INT4 operands (activations and weights alike) are held as E2M3 (fp6) patterns of code / 8 -- exact
+ * for every code in [-15, 15]; the pattern is the sign bit and the 4-bit magnitude -- in "fragments": one operand of the fp6 matrix instruction, 32 rows x
  * one 64-wide k-group = 1536 bytes.  Slot s = row + 32 * half (half: which 32 of the 64 codes) owns a
  * 192-bit string, code j of its half in bits [6 j, 6 j + 6); the first 16 bytes of the string lie at
  * byte 16 s of the fragment, the last 8 at 1024 + 8 s.  Activations: [M_pad/128][K/64][4 fragments]
@@ -59,8 +59,8 @@ const char *svdq_last_error(void);
 int svdq_repack_qweight(const void *src, void *dst, int64_t N, int64_t K, int fp4, void *stream);
 
 /* INT4 wscales bf16 [K/64, N] (reference lane order) -> native [ceil(N/256)][K/64][256 columns] x 8 bytes
- * {bf16(4 * scale), 0, 0, 0}: the operand of the matrix instruction that forms the per-group factor
- * (the 4 undoes the halving of both operands' codes; columns beyond N hold zero).
+ * {bf16(64 * scale), 0, 0, 0}: the operand of the matrix instruction that forms the per-group factor
+ * (the 64 undoes the division by 8 of both operands' codes; columns beyond N hold zero).
  * ceil(N/256) * 256 * (K/64) * 8 bytes.  Replaces packed_wscale_t loads, gemm_base.cuh:474-489. */
 int svdq_repack_wscales(const void *src, void *dst_scales, int64_t N, int64_t K, void *stream);
 

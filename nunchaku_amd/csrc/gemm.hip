@@ -219,18 +219,6 @@ bool acquire_workspace(bool noalloc, int dev, hipStream_t st, size_t zero_bytes,
     return true;
 }
 
-// number of compute units of a device, asked once
-int compute_units(int dev) {
-    static int cached[64] = {0};
-    if (dev < 0 || dev >= 64) return 0;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
 // Into how many parts along K the tiles of an INT4 launch are split when the caller leaves that to the library.
 // Launches with more tiles than compute units are not split: every part parks 128 KB of sums and the last one fetches
 // them all, which only pays while compute units would otherwise stand idle.  Below that, a model of the time in us,

@@ -7,9 +7,9 @@
 // -------------------------------------------------
 //   out[m, n] = sum_g as[m, g] ws[g, n] * sum_{k in g} a[m, k] w[k, n]        (g: 64-wide k-groups)
 // The inner sums are integer products of 4-bit codes.  Both operands are stored as E2M3 patterns of
-// code / 2 (exact for codes -8 .. 15), so that ONE v_mfma_f32_32x32x64_f8f6f4 gives the inner sum of a
+// code / 8 (exact for codes -15 .. 15), so that ONE v_mfma_f32_32x32x64_f8f6f4 gives the inner sum of a
 // 32 x 32 tile for one group, exactly, in fp32, at twice the rate of the INT8 matrix instruction and
-// with no conversion afterwards.  The rank-1 factor as[m, g] * (4 ws[g, n]) of the same tile comes from
+// with no conversion afterwards.  The rank-1 factor as[m, g] * (64 ws[g, n]) of the same tile comes from
 // a second, small matrix instruction (v_mfma_f32_32x32x8bf16_1k with a single non-zero k slot: the
 // product of two bf16 numbers is exact in fp32), and one v_fmac_f32 per accumulator and group adds
 // product * factor to the fp32 accumulator.  Every term is therefore the exactly dequantized product
@@ -27,7 +27,7 @@
 // e % 4 of the 32-column tile.
 //
 // Staging: per k-group a workgroup needs 6 KB of activation fragments, 12 KB of weight fragments,
-// 2 KB of weight scales (stored as {4 s, 0, 0, 0} bf16, the MFMA operand of the factor) and 256 bytes
+// 2 KB of weight scales (stored as {64 s, 0, 0, 0} bf16, the MFMA operand of the factor) and 256 bytes
 // of activation scales; all are contiguous runs in memory and go global -> LDS with asynchronous
 // copies (no registers, no ds_write), three stages deep.  One workgroup barrier per k-group, placed
 // after the last LDS read of the group: behind it the copies of group l + 3 overwrite the stage of
@@ -66,7 +66,7 @@ __device__ inline float16_t mfma_codes(const Frag &w, const Frag &x) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, z, 2, 2, 0, 0, 0, 0);  // E2M3 x E2M3, no block scales
 }
 
-// factor tile 4 ws[n] * as[m]: the weight operand is {4 s, 0, 0, 0} in both half-waves (k slots 0-3 and
+// factor tile 64 ws[n] * as[m]: the weight operand is {64 s, 0, 0, 0} in both half-waves (k slots 0-3 and
 // 4-7), the activation operand carries its scale in k slot 0 and zero in k slot 4, anything finite
 // elsewhere
 __device__ inline float16_t mfma_factor(u32x2_t ws, uint32_t as) {

@@ -198,7 +198,7 @@ struct GemmParams {
 namespace g6 {
 constexpr int BM = 128, BN = 256;  // workgroup tile; 4 waves as 2 x 2, wave tile 64 x 128
 // One stage of the LDS ring holds one k-group of the workgroup's operands:
-//   4 activation fragments | 8 weight fragments | weight scales 256 x {4 s, 0, 0, 0} bf16 |
+//   4 activation fragments | 8 weight fragments | weight scales 256 x {64 s, 0, 0, 0} bf16 |
 //   activation scales 128 x bf16 | zeros (what the upper half-wave reads as its activation scale)
 constexpr int ST_A = 0, ST_W = 4 * FRAG_BYTES, ST_WS = ST_W + 8 * FRAG_BYTES, ST_AS = ST_WS + 256 * 8, ST_Z = ST_AS + 256;
 constexpr int STAGE_BYTES = ST_Z + 128;
@@ -221,7 +221,7 @@ struct Params {
     const uint8_t *act;        // fragments [M_pad/128][K/64][4]
     const uint16_t *ascales;   // bf16 [K/64][M_pad]
     const uint8_t *wgt;        // fragments [ceil(N/256)][K/64][8]
-    const uint8_t *wscales;    // [ceil(N/256)][K/64][256] x {bf16 4 * scale, 0, 0, 0}
+    const uint8_t *wscales;    // [ceil(N/256)][K/64][256] x {bf16 64 * scale, 0, 0, 0}
     const uint16_t *bias;      // bf16 [N] or null
     const uint16_t *wcscales;  // bf16 [N] or null
     const float *lora_act;     // fp32 [M_pad][R_up]

@@ -85,7 +85,7 @@ __device__ inline int64_t wscale_src_index(int64_t g, int64_t n, int64_t G) {
 }
 
 // INT4 weight scales as the operand of the GEMM's factor MFMA: [ceil(N/256)][K/64][256 columns] x
-// {bf16(4 s), 0, 0, 0} (the 4 undoes the halving of both operands' codes; exact, a power of two).
+// {bf16(64 s), 0, 0, 0} (the 64 undoes the division by 8 of both operands' codes; exact, a power of two).
 // Columns beyond N hold zero.
 __global__ void repack_wscales_kernel(const uint16_t *__restrict__ src, unsigned long long *__restrict__ dst, int64_t N, int64_t G) {
     const int64_t nblocks = (N + WGT_BLOCK_COLS - 1) / WGT_BLOCK_COLS;
@@ -94,7 +94,7 @@ __global__ void repack_wscales_kernel(const uint16_t *__restrict__ src, unsigned
     const int64_t n = (i / (G * WGT_BLOCK_COLS)) * WGT_BLOCK_COLS + i % WGT_BLOCK_COLS;
     const int64_t g = (i / WGT_BLOCK_COLS) % G;
     unsigned long long v = 0;
-    if (n < N) v = f32_to_bf16_bits(4.0f * bf16_bits_to_f32(src[wscale_src_index(g, n, G)]));
+    if (n < N) v = f32_to_bf16_bits(64.0f * bf16_bits_to_f32(src[wscale_src_index(g, n, G)]));
     dst[i] = v;
 }
 

@@ -35,6 +35,20 @@ inline int check_launch(const char *what) {
     if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "%s: %s (%s)", what, hipGetErrorString(e), hipGetErrorName(e));
     return SVDQ_OK;
 }
+// number of compute units of a device, asked once (0: the query failed)
+inline int compute_units(int dev) {
+    static int cached[64] = {0};
+    if (dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
 #define SVDQ_REQUIRE(cond, ...) \
     do {                        \
         if (!(cond)) return svdq::fail(SVDQ_EINVAL, __VA_ARGS__); \
@@ -94,8 +108,11 @@ constexpr int TILE_BYTES = TILE_ROWS * GROUP_K / 2;  // 1024
 __host__ __device__ inline uint32_t rotl32(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
 
 // INT4 operands of the GEMM (activations and weights alike) are stored as E2M3 (fp6) patterns of
-// code / 2, which is exact for every code in [-8, 15]: the fp6 matrix instruction then multiplies the
-// bare codes at twice the INT8 rate and returns fp32.  A "fragment" is one operand of
+// code / 8, which is exact for every code in [-15, 15]: the fp6 matrix instruction then multiplies the
+// bare codes at twice the INT8 rate and returns fp32.  (Divided by 8 the codes fill the format's
+// subnormals and its first binade, where the spacing is uniform: the pattern is the sign and the 4-bit
+// magnitude as they are, and the hardware's round-to-nearest-even conversion of a real number to the
+// format IS the rounding to the nearest integer code.)  A "fragment" is one operand of
 // v_mfma_f32_32x32x64_f8f6f4: 32 rows x 64 codes (one k-group) = 1536 bytes.  Slot s = row + 32 * half
 // (half = which 32 of the 64 codes) owns the 192-bit string with code j of its half in bits
 // [6 j, 6 j + 6); the first 16 bytes of the string are stored at 16 s, the last 8 at 1024 + 8 s, so that
@@ -106,11 +123,12 @@ __host__ __device__ inline uint32_t rotl32(uint32_t x, int r) { return (x << r) 
 constexpr int FRAG_BYTES = 1536;
 constexpr int ACT_BLOCK_ROWS = 128, WGT_BLOCK_COLS = 256;
 
-// E2M3 pattern of code / 2 for an integer code in [-15, 15] (bias 1, subnormals, no inf / nan):
-// magnitudes 0..3 are (x << 2), 4..7 are 8 + 2 x, 8..15 are 16 + x; the sign is bit 5.
+// E2M3 pattern of code / 8 for an integer code in [-15, 15] (bias 1, subnormals, no inf / nan):
+// magnitudes 0..7 are the subnormals x / 8, 8..15 the first binade 1 + (x - 8) / 8, so the five low bits
+// are x itself; the sign is bit 5.
 __host__ __device__ inline uint32_t int4_code_to_e2m3(int code) {
     const uint32_t x = code < 0 ? -code : code;
-    const uint32_t m = x < 4 ? x << 2 : (x < 8 ? 8 + 2 * x : 16 + x);
+    const uint32_t m = x;
     return m | (code < 0 ? 32u : 0u);
 }
 

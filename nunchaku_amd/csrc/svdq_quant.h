@@ -67,10 +67,12 @@ __device__ inline uint32_t pack8_e2m1(const float (&t)[8]) {
 
 // INT4: one lane holds 32 consecutive elements of a row = half of a 64-group; the other half lives in
 // the lane `partner_xor` away.  The 32 codes of the lane leave as the E2M3
-// patterns of code / 2, 6 bits each, code j in bits [6 j, 6 j + 6) of a 192-bit string (`lo` = bits
+// patterns of code / 8, 6 bits each, code j in bits [6 j, 6 j + 6) of a 192-bit string (`lo` = bits
 // [0, 128), `hi` = the rest).  The hardware conversion takes the even and the odd elements as two
-// sources and interleaves them; dividing the already rounded and clamped integer by its scale operand
-// (2) is exact.
+// sources and interleaves them, divides by its scale operand (8: an exponent change) and rounds to the
+// nearest E2M3 value, ties to even: below 2 the format's values are the multiples of 1 / 8, so this is the
+// rounding of y * r to the nearest integer code (rne_to_int of the reference) and no separate rounding
+// instruction is needed.
 template <bool UNSIGNED>
 __device__ inline void quantize_int4_half_group_e2m3(const float (&y)[32], int partner_xor, u32x4_t &lo, u32x2_t &hi, float &scale) {
     typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
@@ -84,16 +86,22 @@ __device__ inline void quantize_int4_half_group_e2m3(const float (&y)[32], int p
 #pragma unroll
     for (int e = 0; e < 16; e++) {
         if (UNSIGNED) {
-            ev[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e], rcp), 0.0f, 15.0f));
-            od[e] = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e + 1], rcp), 0.0f, 15.0f));
+            ev[e] = __builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e], rcp), 0.0f, 15.0f);
+            od[e] = __builtin_amdgcn_fmed3f(__fmul_rn(y[2 * e + 1], rcp), 0.0f, 15.0f);
         } else {
             // signed codes need no clamp: |y| <= amax and rcp = fl(1 / fl(amax / 7)) give |y * rcp| <= 7 (1 + 2^-21),
             // which rounds to 7 at most (the reference clamps to [-8, 7], which these values never leave)
-            ev[e] = __builtin_rintf(__fmul_rn(y[2 * e], rcp));
-            od[e] = __builtin_rintf(__fmul_rn(y[2 * e + 1], rcp));
+            ev[e] = __fmul_rn(y[2 * e], rcp);
+            od[e] = __fmul_rn(y[2 * e + 1], rcp);
         }
     }
-    const u32x6_t w = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, 2.0f);
+    // The instruction works through its 32 inputs in several passes and writes result words while later inputs are
+    // still to be read: a destination that overlaps the sources anywhere but at the first registers of the first
+    // source comes out wrong in its last words (seen: the last two words when the register allocator placed the
+    // destination across the end of the first source).  The compiler's definition of the instruction does not
+    // say so; the early-clobber constraint below keeps the destination off both sources.
+    u32x6_t w;
+    asm("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(w) : "v"(ev), "v"(od), "s"(8.0f));
     lo = u32x4_t{w[0], w[1], w[2], w[3]};
     hi = u32x2_t{w[4], w[5]};
     scale = s;

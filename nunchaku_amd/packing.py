@@ -51,7 +51,7 @@ def repack_qweight(qweight: torch.Tensor, fp4: bool = False) -> torch.Tensor:
 
 def repack_wscales(wscales: torch.Tensor, fp4: bool = False) -> torch.Tensor:
     """Reference-order group scales -> native.  INT4 (bf16 [K/64, N]): the factor operand
-    ``[ceil(N/256)][K/64][256] x {bf16(4 s), 0, 0, 0}`` as int64 ``[ceil(N/256), K/64, 256]``.
+    ``[ceil(N/256)][K/64][256] x {bf16(64 s), 0, 0, 0}`` as int64 ``[ceil(N/256), K/64, 256]``.
     NVFP4 (fp8 [K/16, N]): fp16 column-normalised ``[K/64][N][4]`` viewed as ``[K/16, N]``, with the
     fp32 per-column factor that undoes the normalisation as ``.colnorm``."""
     nv.require_gpu(wscales, "wscales")
@@ -175,10 +175,10 @@ def act_nbytes_per_row(K: int, fp4: bool = False) -> int:
     return K // 2 if fp4 else K * 3 // 4
 
 
-# E2M3 pattern of code / 2 for code in [-8, 15] (csrc/svdq_common.h, int4_code_to_e2m3), and its inverse
+# E2M3 pattern of code / 8 for code in [-15, 15] (csrc/svdq_common.h, int4_code_to_e2m3), and its inverse
 def _e2m3_of_code(code: int) -> int:
     x = abs(code)
-    m = x << 2 if x < 4 else (8 + 2 * x if x < 8 else 16 + x)
+    m = x  # subnormals x / 8 and the first binade 1 + (x - 8) / 8: the five low bits are the magnitude
     return m | (32 if code < 0 else 0)
 
 
@@ -211,7 +211,7 @@ def _fragments_to_logical(buf: torch.Tensor, rows: int, K: int, block_rows: int)
     bits = np.unpackbits(strings.numpy(), axis=-1, bitorder="little").reshape(*f.shape[:3], 64, 32, 6)
     pat = (bits * np.array([1, 2, 4, 8, 16, 32], dtype=np.uint8)).sum(axis=-1).astype(np.int64)  # [blk, g, frag, slot, 32]
     codes = _E2M3_TO_CODE[torch.from_numpy(pat)]
-    assert (codes != 127).all(), "a pattern that is not code / 2 for any INT4 code"
+    assert (codes != 127).all(), "a pattern that is not code / 8 for any INT4 code"
     # slot = row + 32 * half, element j of a half is column 32 * half + j
     codes = codes.reshape(rows // block_rows, K // 64, nf, 2, 32, 32).permute(0, 2, 4, 1, 3, 5)  # blk, frag, row, g, half, j
     return codes.reshape(rows, K).contiguous().to(buf.device)
@@ -224,10 +224,10 @@ def qweight_to_logical(qweight_native: torch.Tensor) -> torch.Tensor:
 
 
 def wscales_to_logical(wscales_native: torch.Tensor, N: int) -> torch.Tensor:
-    """Native INT4 weight scales (``repack_wscales``) -> fp32 [K/64, N] (the factor 4 taken out again)."""
-    w = wscales_native.cpu()  # int64 [nblocks, G, 256], bf16 bits of 4 * scale in the low 16 bits
+    """Native INT4 weight scales (``repack_wscales``) -> fp32 [K/64, N] (the factor 64 taken out again)."""
+    w = wscales_native.cpu()  # int64 [nblocks, G, 256], bf16 bits of 64 * scale in the low 16 bits
     assert ((w >> 16) == 0).all(), "the upper three 16-bit slots of a scale entry must be zero"
-    v = (w.to(torch.int32) << 16).view(torch.float32) * 0.25
+    v = (w.to(torch.int32) << 16).view(torch.float32) * (1.0 / 64.0)
     return v.permute(1, 0, 2).reshape(w.shape[1], -1)[:, :N].contiguous()
 
 

@@ -11,6 +11,11 @@ cross-compiles gfx950 without a GPU).
   read 4 GiB below its operands (a GPU memory fault that depended on where the allocator had placed the tensors).  The
   generated code is scanned: after an asm statement that writes SCC, nothing may read SCC before something else has
   written it.
+* The 32-input fp6 conversion.  ``v_cvt_scalef32_2xpk16_fp6_f32`` writes result words while it still has inputs to
+  read: with a destination that overlapped its sources across the end of the first one, the last two result words came
+  out wrong on the GPU (one instantiation of the quantize kernel, found by comparing configurations).  The compiler
+  does not know; the source issues the instruction through inline assembly with an early-clobber destination, and the
+  generated code of every kernel that converts is scanned for overlapping registers.
 """
 
 import re
@@ -76,6 +81,34 @@ def scc_live_across_asm(lines):
             i = j
         i += 1
     return bad
+
+
+def fp6_conversions_with_overlap(lines):
+    """Every ``v_cvt_scalef32_2xpk16_fp6_f32`` whose destination registers overlap one of its two 16-register sources."""
+    total, bad = 0, []
+    for n, l in enumerate(lines):
+        if "v_cvt_scalef32_2xpk16_fp6_f32" in l:
+            m = re.search(r"v\[(\d+):(\d+)\], v\[(\d+):(\d+)\], v\[(\d+):(\d+)\]", l)
+            assert m, l
+            d0, d1, a0, a1, b0, b1 = map(int, m.groups())
+            total += 1
+            if not (d1 < a0 or d0 > a1) or not (d1 < b0 or d0 > b1):
+                bad.append((n + 1, l.strip()))
+    return total, bad
+
+
+def test_fp6_conversion_never_overwrites_its_own_inputs():
+    assert fp6_conversions_with_overlap(["\tv_cvt_scalef32_2xpk16_fp6_f32 v[14:19], v[2:17], v[18:33], s52"])[1]  # the form that failed
+    assert not fp6_conversions_with_overlap(["\tv_cvt_scalef32_2xpk16_fp6_f32 v[34:39], v[2:17], v[18:33], s52"])[1]
+    flags = [f for f in nv.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    with tempfile.TemporaryDirectory(prefix="svdq_guard_") as tmp:
+        for src, extra in (("quantize.hip", []), ("gemm6_variant.hip", ["-DSVDQ_VARIANT=1"])):
+            out = Path(tmp) / (src + ".s")
+            res = subprocess.run(["/opt/rocm/bin/hipcc", *flags, *extra, "-S", "--cuda-device-only", str(CSRC / src), "-o", str(out)],
+                                 capture_output=True, text=True)
+            assert res.returncode == 0, res.stderr[-3000:]
+            total, bad = fp6_conversions_with_overlap(out.read_text().splitlines())
+            assert total > 0 and not bad, (src, bad[:3])
 
 
 def test_scanner_finds_a_carry_kept_across_an_asm_add():

@@ -25,7 +25,7 @@ def test_repack_golden_vectors(dev):
     announce("repack golden qweight/wscales/vector/lora N=K=256 R=32")
     qn = packing.repack_qweight(torch.from_numpy(z["qweight"]).to(dev))
     N, K = z["codes"].shape
-    # E2M3 fragments of code / 2, decoded back to one code per element
+    # E2M3 fragments of code / 8, decoded back to one code per element
     assert torch.equal(packing.qweight_to_logical(qn).cpu(), torch.from_numpy(z["codes"]))
 
     ws = packing.repack_wscales(_bf16(z["wscales_packed"]).to(dev))
