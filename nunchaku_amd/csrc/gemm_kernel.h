@@ -6,23 +6,28 @@
 // -------------------------------------------------
 // Every 16-wide k-group carries its own activation scale (per row, E4M3) and weight scale (per column,
 // E4M3).  The block-scaled fp4 matrix instruction takes power-of-two scales per 32 elements only, so
-// both operands are dequantized *in registers* to fp16 -- (code) * (scale) is exact in fp16: an E2M1
-// code has 2 significant bits and an E4M3 scale 4 -- and fed to v_mfma_f32_32x32x16_f16 with fp32
-// accumulation.  The result equals the fp32 dequantize-then-matmul definition up to fp32 summation
-// order; no per-group post-scaling exists.
+// both operands are dequantized to fp16 -- (code) * (scale) is exact in fp16: an E2M1 code has 2
+// significant bits and an E4M3 scale 4 -- and fed to v_mfma_f32_32x32x16_f16 with fp32 accumulation.
+// The result equals the fp32 dequantize-then-matmul definition up to fp32 summation order; no
+// per-group post-scaling exists.
+//
+// Every element is dequantized ONCE per workgroup: thread t owns row m0 + t of the tile's activations
+// and column n0 + t of its weights, fetches their codes and scales of a k-group into registers, converts
+// them (the hardware E2M1 -> fp16 conversion and one packed multiply per pair: 8 instructions per 8
+// codes) and writes the fp16 operands to LDS in the order the matrix instruction reads them; all four
+// waves then take their operands from there.  (The first kernel converted in every wave that used an
+// element, twice per workgroup, and the conversions, not the matrix instructions, set its pace.)
 //
 // Range: activation scales are renormalised per row and weight scales per column by powers of two
 // (largest scale of a row / column moved into [2^10, 2^11)), so the fp16 products never overflow and
 // only contributions 2^-25 below the largest of their row / column can underflow.  The shifts are
 // undone exactly in the epilogue.
 //
-// Dequantization of one word (8 E2M1 patterns): the hardware E2M1 -> fp16 conversion and one packed
-// multiply per pair (8 instructions per 8 codes).  Both operands use the same element-to-slot order, so
-// the contraction pairs equal k.
-//
 // Tiling: workgroup = 4 waves (2 x 2), block tile 256 x 256, wave tile 128 x 128 = 4 x 4 MFMA tiles,
-// 256 fp32 accumulators per lane.  Operand tiles are staged through a 4-deep LDS ring, one k-group
-// per stage; global loads for group g+3 are issued before the math of group g.
+// 256 fp32 accumulators per lane.  Two LDS buffers of fp16 operands alternate, one k-group each, one
+// workgroup barrier per k-group: while the matrix instructions of group g run from one buffer, the
+// codes of group g + 1 (requested a group earlier) are converted into the other and those of group
+// g + 2 are requested.
 #pragma once
 
 #include <type_traits>
@@ -91,15 +96,11 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     int lane = tid & 63, wave = tid >> 6;
     int wm = wave >> 1, wn = wave & 1;
     int r32 = lane & 31, h = lane >> 5;
-    int ca = __builtin_amdgcn_readfirstlane(tid >> 6);
-    uint32_t code_voff = lane * 16, as_voff = lane * 4;  // (the wave's part of the scale offset is in as_base)
     auto refresh_thread_coordinates = [&]() {
         int t = threadIdx.x;
         asm volatile("" : "+v"(t));
         tid = t; lane = t & 63; wave = t >> 6;
         wm = wave >> 1; wn = wave & 1; r32 = lane & 31; h = lane >> 5;
-        ca = __builtin_amdgcn_readfirstlane(t >> 6);
-        code_voff = lane * 16; as_voff = lane * 4;
     };
 
     // ---- persistent workgroups, work split in units of two k-groups ----------------------------
@@ -161,15 +162,15 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     int *rowshift = (int *)(lds + SHIFT_OFF);  // [MAX_BATCH][256] power-of-two renormalisation of the rows
     constexpr uint32_t AS_ELT = 4, BS_ELT = 8;  // bytes of scales per (64-group, row / column)
     const uint32_t as_stride = (uint32_t)p.M_pad * AS_ELT, bs_stride = (uint32_t)p.N * BS_ELT;
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
 
-    // Everything needed to stage one tile's operands.  All base addresses are wave-uniform (they live
-    // in scalar registers); a lane adds a 32-bit offset.
+    // Everything thread t needs to stage its row of activations and its column of weights of one tile: the
+    // addresses of their first k-group (codes: 32 bytes per row and k-group in tiles of 32 rows, 1 KB per tile
+    // and k-group; scales: one word of four e4m3 per row, four fp16 per column and k-group).
     struct TileCtx {
         int tile, gb, ge;  // k-groups [gb, ge) of the tile
         int m0, n0, shift;
         bool col_ok;
-        const uint8_t *a_base[2], *b_base[2], *as_base, *bs_base;
+        const uint8_t *a_ptr, *b_ptr, *as_ptr, *bs_ptr;
     };
     // follow: the segment after the one given by prev_* (the next tile, from its first k-group), without divisions
     auto make_ctx = [&](int sidx, int slot, int tid, bool follow, int prev_tile, int prev_m0, int prev_n0) {
@@ -189,145 +190,158 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             segment(sidx, c.tile, c.gb, c.ge);
             tile_coords(c.tile, c.m0, c.n0);
         }
-        c.shift = rowshift[slot * 256 + tid];  // thread tid stages the scales of row tid
-        c.col_ok = c.n0 + ca * 64 < p.N;  // (N is a multiple of 128: a wave's 64 columns are inside or outside together)
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int t = ca + 4 * j;
-            const int nt0 = c.n0 / 32;
-            const int tb = nt0 + t < ntiles32 ? nt0 + t : ntiles32 - 1;  // clamped: its scales are zero
-            c.a_base[j] = p.act + (size_t)(c.m0 / 32 + t) * kgroups * TILE_BYTES;
-            c.b_base[j] = p.wgt + (size_t)tb * kgroups * TILE_BYTES;
-        }
-        // scale sources: one word of four e4m3 (activations) or four fp16 (weights) per (64-group, row / column)
-        c.as_base = (const uint8_t *)p.ascales + (size_t)(c.m0 + ca * 64) * AS_ELT;  // row m0 + tid = m0 + 64 ca + lane
-        // column n0 + tid = n0 + 64 ca + lane; a wave beyond N reads the last 64 columns instead (its scales are
-        // stored as zero), so that the lane part of the offset is the same everywhere and needs no register
-        c.bs_base = (const uint8_t *)p.wscales + (size_t)(c.col_ok ? c.n0 + ca * 64 : p.N - 64) * BS_ELT;
+        c.shift = rowshift[slot * 256 + tid];  // thread tid stages row tid
+        // (N is a multiple of 128: the columns of a 32-column tile are inside or outside together; a thread beyond N
+        // fetches the last tile's codes instead and converts them with scale zero)
+        c.col_ok = c.n0 + tid < p.N;
+        const int tb = c.n0 / 32 + (tid >> 5) < ntiles32 ? c.n0 / 32 + (tid >> 5) : ntiles32 - 1;
+        c.a_ptr = p.act + (size_t)(c.m0 / 32 + (tid >> 5)) * kgroups * TILE_BYTES + (tid & 31) * 32;
+        c.b_ptr = p.wgt + (size_t)tb * kgroups * TILE_BYTES + (tid & 31) * 32;
+        c.as_ptr = (const uint8_t *)p.ascales + (size_t)(c.m0 + tid) * AS_ELT;
+        c.bs_ptr = (const uint8_t *)p.wscales + (size_t)(c.col_ok ? c.n0 + tid : p.N - 1) * BS_ELT;
         return c;
     };
 
     // ---- staging -----------------------------------------------------------------------------
-    // Code tiles go global -> LDS with asynchronous 16-byte copies (no registers, no ds_write);
-    // the two scale values per thread travel through registers because they are renormalised on the
-    // way.  The main loop works on pairs of k-groups with ONE workgroup barrier per pair (a barrier per
-    // group costs 9 % of the loop in waiting for the slowest wave).  At the top of the pair (l, l+1) the
-    // codes and scales of groups l+3 and l+4 are requested; they go into the stages of groups l-1 and l,
-    // which nobody reads any more (group l's operands were taken into registers during group l-1, before
-    // the previous barrier).  The pair itself reads groups l+1 and l+2 from LDS, which were complete at
-    // the previous barrier.  At the end of the pair every wave waits for its own requests (vmcnt(0):
-    // they have had two group times to land), stores the two sets of scales and meets the others at the
-    // barrier.  The loop's vector-memory requests come from volatile asm: the compiler neither reorders
-    // them nor adds waits of its own for them.
-    // (l counts the k-groups of the segment; the stage is l % STAGES, the source group c.gb + l)
-    auto issue_codes = [&](const TileCtx &c, int l) {  // 4 vector-memory operations
-        const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;  // surplus copies at the tail are never consumed
-        const uint32_t dst = lds_base + (l % STAGES) * STAGE_BYTES + ca * TILE_BYTES;
-        const uint32_t voff = (uint32_t)gc * TILE_BYTES + code_voff;
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :: "s"(dst + STAGE_A + 4 * j * TILE_BYTES), "v"(voff), "s"(c.a_base[j]) : "memory", "m0");
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :: "s"(dst + STAGE_B + 4 * j * TILE_BYTES), "v"(voff), "s"(c.b_base[j]) : "memory", "m0");
-        }
+    // One k-group of a thread's row and column on their way from memory to LDS: 64 + 64 codes and their scales.
+    // Ordinary loads: the compiler tracks the registers they write and places the waits itself.
+    struct Raw {
+        u32x4_t a[2], b[2];
+        uint32_t as;
+        u32x2_t bs;
     };
-    // (ordinary loads: the compiler tracks the registers they write and places the waits for them itself.
-    // They are issued AFTER the asynchronous copies of the same groups, which the compiler does not count:
-    // its "all but the n newest requests" waits then cover the older copies too and never wait for less
-    // than intended.)
-    auto issue_scales = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {  // 2 vector-memory operations
-        const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
-        ra = *(const uint32_t *)(c.as_base + ((uint32_t)gc * as_stride + as_voff));
-        rb = *(const u32x2_t *)(c.bs_base + ((uint32_t)gc * bs_stride + as_voff * 2));
+    // (l counts the k-groups of the segment; requests past the end of K repeat the last group and are never used)
+    auto load_raw = [&](const TileCtx &c, int l, Raw &r) {
+        const uint32_t gc = (uint32_t)(c.gb + l < kgroups ? c.gb + l : kgroups - 1);
+        const u32x4_t *ap = (const u32x4_t *)(c.a_ptr + gc * TILE_BYTES), *bp = (const u32x4_t *)(c.b_ptr + gc * TILE_BYTES);
+        r.a[0] = ap[0];
+        r.a[1] = ap[1];
+        r.b[0] = bp[0];
+        r.b[1] = bp[1];
+        r.as = *(const uint32_t *)(c.as_ptr + gc * as_stride);
+        r.bs = *(const u32x2_t *)(c.bs_ptr + gc * bs_stride);
     };
-    auto store_scales = [&](const TileCtx &c, int g, uint32_t ra, u32x2_t rb) {
-        // (row / column tid of the stage tables, addressed through the lane offset that is live anyway:
-        // the main loop has no register to spare for another address)
-        uint8_t *base = lds + (g % STAGES) * STAGE_BYTES + ca * 1024 + code_voff;
-        u32x4_t pa, pb;
+    // Words 2 ks and 2 ks + 1 of the thread's row and of its column (16-group ks of the k-group) -> fp16 -> the
+    // operand buffer: word w holds the codes of k = 8 w .. 8 w + 7, which are one lane's operand of the matrix
+    // instruction (step w / 2, half w % 2); a wave's 64 threads write 64 consecutive 16-byte slots per word.
+    // `which`: 0, 1 the two words of the row, 2, 3 those of the column.
+    auto group_scales = [&](const TileCtx &c, const Raw &r, int ks, half2_t &sa2, half2_t &sb2) {
+        // e4m3 -> fp16 with the row's shift, without branches (a branch would end the scheduling region in which the
+        // conversions are interleaved with the matrix instructions)
+        const uint32_t e8 = (r.as >> (8 * ks)) & 0x7Fu, ex = e8 >> 3;
+        const _Float16 sa = (_Float16)ldexpf((float)((e8 & 7u) | (ex ? 8u : 0u)), (int)(ex ? ex : 1u) - 10 + c.shift);
+        const uint32_t hb = c.col_ok ? (r.bs[ks >> 1] >> (16 * (ks & 1))) & 0xFFFFu : 0u;
+        sa2 = half2_t{sa, sa};
+        sb2 = as_half2(hb | (hb << 16));
+    };
+    auto convert_word = [&](const Raw &r, uint32_t buf, int ks, int which, half2_t sa2, half2_t sb2, int tid) {
+        uint8_t *base = lds + buf * OPBUF_BYTES + (tid >> 5) * (4 * 2 * 32 * 16) + (tid & 31) * 16 + (ks * 2 + (which & 1)) * 512;
+        const int w = 2 * ks + (which & 1);
+        if (which < 2) *(half8_t *)base = dequant_word_fp4(r.a[w >> 2][w & 3], sa2);
+        else *(half8_t *)(base + OP_BYTES) = dequant_word_fp4(r.b[w >> 2][w & 3], sb2);
+    };
+    auto convert_store = [&](const TileCtx &c, const Raw &r, uint32_t buf, int ks, int tid) {
+        half2_t sa2, sb2;
+        group_scales(c, r, ks, sa2, sb2);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const _Float16 sa = (_Float16)ldexpf(e4m3_to_f32((ra >> (8 * j)) & 0x7Fu), c.shift);
-            pa[j] = as_u32(half2_t{sa, sa});
-            const uint32_t hb = c.col_ok ? (rb[j >> 1] >> (16 * (j & 1))) & 0xFFFFu : 0u;
-            pb[j] = hb | (hb << 16);
-        }
-        *(u32x4_t *)(base + STAGE_AS) = pa;
-        *(u32x4_t *)(base + STAGE_BS) = pb;
+        for (int which = 0; which < 4; which++) convert_word(r, buf, ks, which, sa2, sb2, tid);
     };
 
     float16_t acc[4][4];
     int coltab_n0 = -1;  // first column of the tile whose column tables are in LDS (wave-uniform)
-    uint32_t sa_e, sa_o;  // scale registers in flight: first / second group of the pair being requested
-    u32x2_t sb_e, sb_o;
-    uint32_t s0a, s1a, s2a;  // scales of groups 0..2 of a tile whose first stages are being fetched
-    u32x2_t s0b, s1b, s2b;
-    // first stages of a tile: scales and codes of groups 0..2.  These scale loads are ordinary loads, not
-    // asm: they may stay in flight across a whole epilogue, and only loads the compiler knows about are
-    // safe against register copies and spills made before the data has arrived.
-    auto load_scales_plain = [&](const TileCtx &c, int l, uint32_t &ra, u32x2_t &rb) {
-        const int gc = c.gb + l < kgroups ? c.gb + l : kgroups - 1;
-        ra = *(const uint32_t *)(c.as_base + (gc * as_stride + as_voff));
-        rb = *(const u32x2_t *)(c.bs_base + (gc * bs_stride + lane * BS_ELT));
-    };
-    auto issue_first_stages = [&](const TileCtx &c) {
-        load_scales_plain(c, 0, s0a, s0b);
-        load_scales_plain(c, 1, s1a, s1b);
-        load_scales_plain(c, 2, s2a, s2b);
-        issue_codes(c, 0);
-        issue_codes(c, 1);
-        issue_codes(c, 2);
-    };
+    Raw rawa, rawb, rawc, rawd;  // codes on their way: `rawc`, `rawd` are converted next, the other two are requests in flight
 
-    // Software pipeline over the 16-wide MFMA steps (4 per k-group): while the 16 MFMAs of a step run,
-    // the VALU dequantizes the operands of the next step, so a wave never waits on its own
-    // conversions.  raw_* hold the packed codes and scales of the current k-group, *_n of the next.
-    u32x4_t araw[4], braw[4], araw_n[4], braw_n[4];
-    u32x2_t asc[4], bsc[4], asc_n[4], bsc_n[4];
-    half8_t a0[4], b0[4], a1[4], b1[4];
-    auto read_raw = [&](int st, u32x4_t (&ar)[4], u32x4_t (&br)[4], u32x2_t (&as)[4], u32x2_t (&bs)[4]) {
-        const uint8_t *base = lds + st * STAGE_BYTES;
+    // The arithmetic of one k-group: four steps of 16 matrix instructions on the operands in buffer `buf`; the
+    // operands of a step are fetched during the step before; between the matrix instructions the group `rc` is
+    // converted into the other buffer, one 16-group per step.
+    half8_t opa[2][4], opb[2][4];
+    auto read_a = [&](uint32_t buf, int ks, int t, half8_t &a) {
+        a = *(const half8_t *)(lds + buf * OPBUF_BYTES + (ks * 2 + h) * 512 + r32 * 16 + (wm * 4 + t) * (4 * 2 * 32 * 16));
+    };
+    auto read_b = [&](uint32_t buf, int ks, int t, half8_t &b) {
+        b = *(const half8_t *)(lds + buf * OPBUF_BYTES + OP_BYTES + (ks * 2 + h) * 512 + r32 * 16 + (wn * 4 + t) * (4 * 2 * 32 * 16));
+    };
+    // One piece (of six) of a k-group's requests: a thread's two 16-byte halves of its row's codes, the same of its
+    // column's, the row's scales, the column's scales.
+    auto load_piece = [&](const TileCtx &c, int l, Raw &r, int piece) {
+        const uint32_t gc = (uint32_t)(c.gb + l < kgroups ? c.gb + l : kgroups - 1);
+        if (piece == 0) r.a[0] = *(const u32x4_t *)(c.a_ptr + gc * TILE_BYTES);
+        if (piece == 1) r.a[1] = *(const u32x4_t *)(c.a_ptr + gc * TILE_BYTES + 16);
+        if (piece == 2) r.b[0] = *(const u32x4_t *)(c.b_ptr + gc * TILE_BYTES);
+        if (piece == 3) r.b[1] = *(const u32x4_t *)(c.b_ptr + gc * TILE_BYTES + 16);
+        if (piece == 4) r.as = *(const uint32_t *)(c.as_ptr + gc * as_stride);
+        if (piece == 5) r.bs = *(const u32x2_t *)(c.bs_ptr + gc * bs_stride);
+    };
+    // A k-group is four steps of 16 k; a step is four quarters, each in this order and fenced from the next (left
+    // alone, the scheduler gathers the matrix instructions in long runs and the conversions in others, and the two
+    // pipes take turns instead of working side by side): two operand tiles of the next step are requested, one word
+    // of `rc` is converted and stored, four matrix instructions are issued with the conversion between them.  A wave
+    // is alone on its SIMD, so whatever stands in front of a matrix instruction is lost time; therefore also:
+    //   - the scales of a step's 16-group are prepared during the step before (those of the next group's first step
+    //     during this group's last, from `rc_next`);
+    //   - the requests for later groups (LOADS: both groups the iteration asks for) are issued one per quarter;
+    //   - a second barrier in the middle of the group publishes the first half of the other buffer, so that the
+    //     operands of the next group's first step can be fetched during this group's last step instead of behind
+    //     the barrier that ends the group; neither barrier waits for the LDS queue to drain (see below).
+    // (the group behind the last one of a segment is converted too, into the buffer nobody reads any more: a
+    // condition would split the body into basic blocks)
+    half2_t sa2, sb2;  // scales of the 16-group converted next
+    auto group = [&](auto LOADS_T, const TileCtx &c, uint32_t buf, const Raw &rc, const Raw &rc_next, int l_load, Raw &ld0, Raw &ld1) {
+        constexpr bool LOADS = decltype(LOADS_T)::value;
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            ar[t] = *(const u32x4_t *)(base + STAGE_A + (wm * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
-            br[t] = *(const u32x4_t *)(base + STAGE_B + (wn * 4 + t) * TILE_BYTES + r32 * 32 + h * 16);
-            as[t] = *(const u32x2_t *)(base + STAGE_AS + (wm * 128 + t * 32 + r32) * 16 + h * 8);
-            bs[t] = *(const u32x2_t *)(base + STAGE_BS + (wn * 128 + t * 32 + r32) * 16 + h * 8);
+        for (int ks = 0; ks < 4; ks++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int nq = ks * 4 + q;  // quarter of the group
+                half2_t sa2n = sa2, sb2n = sb2;
+                if (q == 3) group_scales(c, ks < 3 ? rc : rc_next, (ks + 1) & 3, sa2n, sb2n);
+                if (LOADS && nq < 12) load_piece(c, l_load + nq / 6, nq < 6 ? ld0 : ld1, nq % 6);
+                // (the next step's first quarter needs all four weight tiles and the first activation tile: the
+                // weight tiles are requested first, every operand at least two quarters before its use)
+                const uint32_t rbuf = ks < 3 ? buf : buf ^ 1;
+                if (q < 2) {
+                    read_b(rbuf, (ks + 1) & 3, 2 * q, opb[(ks + 1) & 1][2 * q]);
+                    read_b(rbuf, (ks + 1) & 3, 2 * q + 1, opb[(ks + 1) & 1][2 * q + 1]);
+                } else {
+                    read_a(rbuf, (ks + 1) & 3, 2 * q - 4, opa[(ks + 1) & 1][2 * q - 4]);
+                    read_a(rbuf, (ks + 1) & 3, 2 * q - 3, opa[(ks + 1) & 1][2 * q - 3]);
+                }
+                convert_word(rc, buf ^ 1, ks, q, sa2, sb2, tid);
+#pragma unroll
+                for (int nt = 0; nt < 4; nt++)
+                    acc[q][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(opb[ks & 1][nt], opa[ks & 1][q], acc[q][nt], 0, 0, 0);
+                if (LOADS && nq < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                if (q == 3) {  // (with the preparation of the next step's scales)
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                } else {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                sa2 = sa2n;
+                sb2 = sb2n;
+                // The two barriers of a group stand one quarter BEHIND the stores they publish (the end of the previous
+                // group, the end of step 1): a wave's LDS operations complete in order, so waiting until only this
+                // quarter's three (two fetches, one store) are outstanding proves the earlier stores complete without
+                // draining the queue of fetches that keeps the matrix instructions fed.  What this quarter stores
+                // belongs to the half that the next barrier publishes; nobody fetches what a wave one quarter ahead
+                // overwrites (that region was last fetched a whole group earlier).
+                if (q == 0 && (ks == 0 || ks == 2)) asm volatile("s_waitcnt lgkmcnt(3)\n\ts_barrier" ::: "memory");
+            }
         }
     };
-#define SVDQ_CONVERT(AR, BR, AS, BS, I, A, B)                                                             \
-    _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                       \
-        /* word I of the lane's 32 codes lies in 16-group 2h + I/2 */                                     \
-        A[t] = dequant_word_fp4(AR[t][I], as_half2(AS[t][(I) >> 1]));                                      \
-        B[t] = dequant_word_fp4(BR[t][I], as_half2(BS[t][(I) >> 1]));                                      \
-    }
-#define SVDQ_MFMA(A, B)                                                                                   \
-    _Pragma("unroll") for (int mt = 0; mt < 4; mt++) _Pragma("unroll") for (int nt = 0; nt < 4; nt++)     \
-        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[nt], A[mt], acc[mt][nt], 0, 0, 0);
-    // the arithmetic of one k-group: 64 MFMAs and the conversions for the next 64
-#define SVDQ_GROUP(G)                                                                                     \
-    {                                                                                                     \
-        SVDQ_CONVERT(araw, braw, asc, bsc, 1, a1, b1)                                                     \
-        SVDQ_MFMA(a0, b0)                                                                                 \
-        SVDQ_CONVERT(araw, braw, asc, bsc, 2, a0, b0)                                                     \
-        SVDQ_MFMA(a1, b1)                                                                                 \
-        read_raw(((G) + 1) % STAGES, araw_n, braw_n, asc_n, bsc_n);                                       \
-        SVDQ_CONVERT(araw, braw, asc, bsc, 3, a1, b1)                                                     \
-        SVDQ_MFMA(a0, b0)                                                                                 \
-        SVDQ_CONVERT(araw_n, braw_n, asc_n, bsc_n, 0, a0, b0)                                             \
-        SVDQ_MFMA(a1, b1)                                                                                 \
-        _Pragma("unroll") for (int t = 0; t < 4; t++) {                                                   \
-            araw[t] = araw_n[t]; braw[t] = braw_n[t]; asc[t] = asc_n[t]; bsc[t] = bsc_n[t];               \
-        }                                                                                                 \
-        /* an MFMA takes two issue slots, every other instruction one; 8 passes cover six of them */      \
-        _Pragma("unroll") for (int k = 0; k < 32; k++) {                                                  \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
-            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
-            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                            \
-        }                                                                                                 \
-    }
 
   for (int batch0 = 0; batch0 < nseg; batch0 += MAX_BATCH) {
     const int nbatch = nseg - batch0 < MAX_BATCH ? nseg - batch0 : MAX_BATCH;
@@ -365,12 +379,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     __syncthreads();
 
     TileCtx cur = make_ctx(batch0, 0, threadIdx.x, false, 0, 0, 0);
-    issue_first_stages(cur);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    store_scales(cur, 0, s0a, s0b);
-    store_scales(cur, 1, s1a, s1b);
-    store_scales(cur, 2, s2a, s2b);
-    __syncthreads();
 
    for (int ti = 0; ti < nbatch; ti++) {
     const bool have_next = ti + 1 < nbatch;
@@ -382,30 +390,30 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    read_raw(0, araw, braw, asc, bsc);
-    SVDQ_CONVERT(araw, braw, asc, bsc, 0, a0, b0)
-    // the first iteration refills stage 0, which every wave has to have read by then (inside the loop the
-    // barrier that ends an iteration orders the reads of a stage before its refill)
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // Groups 0 to 2 of the segment are requested, group 0 converted into buffer 0 (the previous tile's epilogue is
+    // done with the LDS it shares with the buffers: every tile ends with a barrier).  An iteration multiplies groups
+    // l and l + 1 (buffers 0 and 1) and converts groups l + 1 and l + 2 from `rawc` and `rawd`; groups l + 3 and
+    // l + 4 are requested during its first group into `rawa` and `rawb` and handed over at its end.  Segments are an
+    // even number of groups long.
+    load_raw(cur, 0, rawa);
+    load_raw(cur, 1, rawc);
+    load_raw(cur, 2, rawd);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) convert_store(cur, rawa, 0, ks, tid);
+    group_scales(cur, rawc, 0, sa2, sb2);
     __syncthreads();
-    // The compiler cannot see the waits issued from asm.  A wait through the builtin, which its
-    // bookkeeping understands, tells it that none of its own loads is in flight when the loop starts
-    // (the hand-over has waited for everything already).
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt unconstrained
-    const int seg_len = cur.ge - cur.gb;  // even: segments begin and end on units of two k-groups
-    for (int l = 0; l < seg_len; l += 2) {
-        issue_codes(cur, l + 3);
-        issue_codes(cur, l + 4);
-        issue_scales(cur, l + 3, sa_e, sb_e);
-        issue_scales(cur, l + 4, sa_o, sb_o);
-        SVDQ_GROUP(l)
-        SVDQ_GROUP(l + 1)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the copies (the compiler waits for the scale loads itself)
-        store_scales(cur, l + 3, sa_e, sb_e);
-        store_scales(cur, l + 4, sa_o, sb_o);
-        __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        read_b(0, 0, t, opb[0][t]);
+        read_a(0, 0, t, opa[0][t]);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const int seg_len = cur.ge - cur.gb;
+    for (int l = 0; l < seg_len; l += 2) {
+        group(std::true_type{}, cur, 0, rawc, rawd, l + 3, rawa, rawb);   // group l; group l + 1 -> buffer 1
+        group(std::false_type{}, cur, 1, rawd, rawa, 0, rawa, rawb);      // group l + 1; group l + 2 -> buffer 0
+        rawc = rawa;
+        rawd = rawb;
+    }
     // pin the accumulators in the accumulation registers across the loop exit: without this the
     // register allocator may place the 256 copies into ordinary registers inside the loop body
     asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]),
@@ -566,14 +574,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
             }
         }
     }
-    // everything requested so far has arrived before the next tile's first stages are requested: a
-    // wait on a later request would otherwise also wait for everything issued in between
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_wave_barrier();
-    // first stages of the next tile: in flight while this tile's epilogue runs (the LDS stages are
-    // free, the epilogue works in its own slab)
-    if (have_next) issue_first_stages(nxt);
-
     // reciprocal smoothing factors of the next layer for the 32 columns this lane quantizes
     // (work item of the quantizing pass: row = item / 4, 32-column quarter = item % 4 = lane % 4)
     float nrs[32];
@@ -835,27 +835,10 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         slab_epilogue(std::integral_constant<int, 2>{}, std::true_type{});
         slab_epilogue(std::integral_constant<int, 3>{}, std::true_type{});
     }
-    if (have_next) {
-        // The code copies of the next tile must have landed.  s_waitcnt vmcnt(n) returns once at most n
-        // requests are outstanding, so it proves that the copies are complete only if at least n
-        // requests were issued after them.  That is known for an interior tile of the plain variant:
-        // each wave issues its 32 output stores (none is skipped, no lane is out of range), and leaving
-        // those in flight lets them drain while the next tile starts.  Everywhere else: wait for all.
-        if (!NEXT && run_epilogue && interior)
-            asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
-        else
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        cur = nxt;
-        store_scales(cur, 0, s0a, s0b);
-        store_scales(cur, 1, s1a, s1b);
-        store_scales(cur, 2, s2a, s2b);
-    }
+    if (have_next) cur = nxt;
     __syncthreads();
    }  // tiles of the batch
   }    // batches
-#undef SVDQ_GROUP
-#undef SVDQ_CONVERT
-#undef SVDQ_MFMA
 }
 
 

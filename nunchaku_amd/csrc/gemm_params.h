@@ -11,20 +11,21 @@ namespace svdq {
 constexpr int MAX_RANK = 1024;
 
 constexpr int BM = 256, BN = 256;
-constexpr int STAGES = 4;
-// per stage: 8 KB A codes, 8 KB B codes, then 16 bytes of packed fp16 scale pairs per row / column:
-// INT4 {16s,16s} {-24s,-24s} (8 bytes used; -16s for unsigned codes); NVFP4 one {s,s} pair for each
-// of the four 16-groups
-constexpr int STAGE_A = 0, STAGE_B = 8192, STAGE_AS = 16384, STAGE_BS = 16384 + 4096;
-constexpr int STAGE_BYTES = 16384 + 8192;
+// NVFP4 kernel: the operands of one k-group (64 wide) as fp16, dequantized once per workgroup: per operand
+// [8 tiles of 32 rows][4 steps of 16 k][2 halves of 8 k][32 rows] x 16 bytes = 32 KB (a wave's fetch of one matrix
+// instruction's operand is 1 KB contiguous), activations then weights; two such buffers alternate.
+constexpr int OP_BYTES = 8 * 4 * 2 * 32 * 16;    // one operand of one k-group
+constexpr int OPBUF_BYTES = 2 * OP_BYTES;          // activations + weights
 constexpr int OUT_LD = 136;                // bf16 elements per row of the store-staging slab (128 + pad)
 constexpr int MAX_BATCH = 8;                       // tiles whose row shifts are tabulated at once
-constexpr int SLAB_OFF = STAGES * STAGE_BYTES;     // 4 waves x (32 rows x OUT_LD bf16): epilogue staging
-constexpr int SHIFT_OFF = SLAB_OFF + 4 * 32 * OUT_LD * 2;  // int [MAX_BATCH][256] row renormalisation shifts
+constexpr int SLAB_OFF = 0;                        // 4 waves x (32 rows x OUT_LD bf16): epilogue staging, in the operand buffers' place
+static_assert(4 * 32 * OUT_LD * 2 <= 2 * OPBUF_BYTES, "the epilogue's slabs reuse the operand buffers");
+constexpr int SHIFT_OFF = 2 * OPBUF_BYTES;                 // int [MAX_BATCH][256] row renormalisation shifts
 constexpr int TAB_OFF = SHIFT_OFF + MAX_BATCH * 256 * 4;   // 4 waves x float [2][128]: column factors and biases
 constexpr int FLAG_OFF = TAB_OFF + 4 * 1024;               // one word: a thread's reading of an arrival counter, for all
 constexpr int NORMW_OFF = FLAG_OFF + 16;                   // 4 waves x float [128]: RMS-norm weights of the wave's head
 constexpr int LDS_BYTES = NORMW_OFF + 4 * 512;
+static_assert(LDS_BYTES <= 160 * 1024, "one workgroup per compute unit");
 constexpr int NORM_TARGET_EXP = 10;
 
 
