@@ -154,8 +154,9 @@ typedef struct svdq_gemm_args {
     const void *wscales;    /* native scales (svdq_repack_wscales / _wmscales)                      */
     const float *colnorm;   /* NVFP4: fp32 [N] from svdq_repack_wmscales; INT4: ignored, may be NULL */
     const void *bias;       /* bf16 [N] channel order, or NULL                                      */
-    const void *wcscales;   /* bf16 [N] channel order, or NULL; NVFP4: no element may be zero (the
-                               low-rank term is added in units of the column factor)                */
+    const void *wcscales;   /* bf16 [N] channel order, or NULL; NVFP4 with a low-rank branch: no element may
+                               be zero (the low-rank term is added in units of the column factor); the
+                               Python wrappers check it once per tensor, a caller of the C ABI must     */
     const float *lora_act_in; /* fp32 [M_pad, R_up] row-major, or NULL                              */
     const void *lora_up;    /* bf16 [N, R_up] (svdq_repack_lora_up), or NULL                        */
     const float *lora_scales; /* HOST pointer, ceil(R_up/16) floats, or NULL for all ones           */

@@ -181,6 +181,8 @@ class SVDQW4A4Linear(nn.Module):
                 "bias": None if self.bias is None else packing.repack_vector(self.bias.data),
                 "wcscales": None if self.wcscales is None else packing.repack_vector(self.wcscales.data),
             }
+            if fp4 and self.rank:
+                packing.require_nonzero(self._native["wcscales"], "wcscales")
         return self._native
 
     # ---- low-rank hot swap ---------------------------------------------------------------------

@@ -169,6 +169,8 @@ def svdq_gemm_w4a4(
     wsc_n = packing.native(wscales, "wscales", fp4)
     bias_n = packing.native(bias, "vector")
     wcs_n = packing.native(wcscales, "vector")
+    if fp4 and lora_up is not None:
+        packing.require_nonzero(wcs_n, "wcscales")
     up_n = packing.native(lora_up, "lora_up")
     nsm_n = packing.native(smooth_factor, "smooth_rcp") if qout is not None else None
     ndown_n = packing.native(lora_down, "lora_down")

@@ -165,6 +165,18 @@ def native(t: torch.Tensor | None, kind: str, fp4: bool = False) -> torch.Tensor
     return out
 
 
+def require_nonzero(t: torch.Tensor | None, what: str) -> None:
+    """Raise if a native per-channel vector holds a zero.  The NVFP4 GEMM adds the low-rank term in units of
+    the column factor (column normalisation x alpha x wcscales), i.e. divides by it: a zero there would silently
+    drop the term.  Checked once per tensor object (the check reads the tensor back: one synchronisation)."""
+    if t is None or getattr(t, "_svdq_nonzero", False):
+        return
+    if bool((t == 0).any()):
+        raise ValueError(f"{what} holds a zero: the NVFP4 kernel adds the low-rank term in units of the per-channel factor "
+                         "and cannot divide by it (the reference multiplies only)")
+    t._svdq_nonzero = True
+
+
 # ---------------------------------------------------------------------------------------------
 # logical views of the kernels' private 4-bit tile layout (for tests and debugging)
 # ---------------------------------------------------------------------------------------------

@@ -63,6 +63,19 @@ def test_nvfp4_layer_end_to_end(dev):
     check_output(y, ref.forward_quant(codes, scales, lora)[:M])
 
 
+def test_nvfp4_zero_per_channel_scale_is_refused(dev):
+    """The NVFP4 kernel divides the low-rank term by the per-channel factor: a zero in wcscales is refused when the
+    layer's tensors are converted, instead of silently dropping the term for that channel."""
+    M, K, N, R = 256, 256, 256, 16
+    announce("nvfp4 layer with a zero in wcscales")
+    layer = synth.make_layer(N, K, R, seed=32, fp4=True)
+    layer.wcscales = torch.ones(N, dtype=torch.bfloat16)
+    layer.wcscales[5] = 0.0
+    m = make_module(layer, dev)
+    with pytest.raises(ValueError, match="wcscales"):
+        m(synth.make_activations(M, K, seed=32).to(dev).view(1, M, K))
+
+
 @pytest.mark.parametrize("M,K1,N1,R", [(256, 256, 512, 16), (2304, 256, 7680, 32), (3072, 256, 10752, 32)])
 def test_nvfp4_fused_mlp_epilogue(dev, M, K1, N1, R):
     """NVFP4 GEMM producing the next layer's NVFP4 input (no shift, signed patterns).  The second shape has 270 tiles,
