@@ -34,9 +34,22 @@ WORKLOADS = {
     "flux_single_out_nvfp4": dict(M=4608, K=15360, N=3072, R=32, seed=3, fp4=True),
 }
 INT8_PEAK_TOPS = 5000.0  # MI355X dense INT8 MFMA, the peak the metric is quoted against
-# HBM-side bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
-# read for a device copy of known size (profiles/gemm6_kernel_*.md); only known for the profiled workload
-PROFILED_GEMM_TRAFFIC_BYTES = {"flux_mlp_fc1": (2.0 * 144340 + 1.0 * 110590) * 1024}
+# HBM-side bytes per GEMM launch: rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch, mean of the launches of
+# `bench.py --only gemm --workload W --steps 3`), each scaled by what the same counter reads for a device copy of known size
+# (`bench.py --only copy`: FETCH_SIZE reads 131085 for 262144 KiB, factor 2.0; WRITE_SIZE reads 262144, factor 1.0).  The
+# commands and the readings are in profiles/w4a4_gemm_hbm_traffic_all_workloads.md; a workload that is not in the table (a
+# custom --shape, --qkv-rope) reports null.
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+PROFILED_GEMM_FETCH_WRITE_KIB = {
+    "flux_mlp_fc1": (143432.6, 110593.0),
+    "flux_qkv": (103458.7, 82944.7),
+    "flux_mlp_fc2": (154337.3, 27648.0),
+    "qwen_batched_r128": (696300.5, 442369.8),
+    "c1_small": (12820.6, 10755.0),
+    "flux_single_nvfp4": (151611.5, 215470.7),
+    "flux_single_out_nvfp4": (122092.9, 31320.1),
+}
+PROFILED_GEMM_TRAFFIC_BYTES = {w: (FETCH_SCALE * f + WRITE_SCALE * wr) * 1024 for w, (f, wr) in PROFILED_GEMM_FETCH_WRITE_KIB.items()}
 HBM_PEAK_GBS = 8000.0
 
 
@@ -82,13 +95,17 @@ def main():
     ap.add_argument("--qkv-rope", action="store_true",
                     help="time the GEMM with the RMS-norm + rotary epilogue of fused_qkv_norm_rottary (workload flux_qkv); "
                          "the CPU comparison is skipped")
-    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "awq-gemv", "fused-mlp", "litela"], default=None,
+    ap.add_argument("--only", choices=["gemm", "quantize", "copy", "awq-gemv", "fused-mlp", "litela", "power"], default=None,
                     help="profiling aid: launch only one of the two kernels in the timed loops (prints no JSON); "
                          "'copy' launches a plain device copy of 256 MiB, the yardstick for the HBM traffic counters; "
                          "'awq-gemv' times the AWQ W4A16 GEMV at the modulation shape (1 row, K=3072, N=18432); "
                          "'fused-mlp' times fused_gelu_mlp on the FLUX MLP pair (M=4608, 3072 -> 12288 -> 3072); "
                          "'litela' times the linear-attention pair (QKV projection with the q / vk epilogue, then vk times q) at "
-                         "4096 tokens, K=2304, 72 heads of 32")
+                         "4096 tokens, K=2304, 72 heads of 32; "
+                         "'power' times the workload's GEMM kernel launched back to back on its synthetic activations and on all-zero "
+                         "activations (same weights, same launches), and the vendor library's dense GEMM of the same "
+                         "M, K, N (fp16 and bf16 through torch.matmul, int8 through torch._int_mm) on random and on zero operands: "
+                         "a kernel whose time follows the operands' bit activity at equal work runs against the power limit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -234,6 +251,93 @@ def main():
         svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"], fp4=fp4)
         gemm()
 
+    if args.only == "power":
+        import re
+        import subprocess
+        import threading
+
+        class Sensors:
+            """Shader clock and package power as `rocm-smi` reports them, sampled by a thread while a timed loop runs."""
+
+            def __init__(self):
+                self.samples, self.stop = [], threading.Event()
+
+            def _run(self):
+                while not self.stop.is_set():
+                    try:
+                        txt = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--json"], capture_output=True, text=True, timeout=10).stdout
+                        card = next(iter(json.loads(txt).values()))
+                        clk = [float(re.search(r"(\d+)\s*Mhz", v, re.I).group(1)) for k, v in card.items() if k.lower().startswith("sclk") and re.search(r"(\d+)\s*Mhz", str(v), re.I)]
+                        pw = [float(v) for k, v in card.items() if "power" in k.lower() and re.fullmatch(r"[\d.]+", str(v).strip())]
+                        self.samples.append((clk[0] if clk else None, pw[0] if pw else None))
+                    except Exception:  # no tool, no permission, another output format: the timings stand without it
+                        return
+
+            def __enter__(self):
+                self.thread = threading.Thread(target=self._run, daemon=True)
+                self.thread.start()
+                return self
+
+            def __exit__(self, *exc):
+                self.stop.set()
+                self.thread.join(timeout=15)
+
+            def text(self):
+                clk = [c for c, _ in self.samples[1:] if c]  # (the first sample may predate the loop)
+                pw = [w for _, w in self.samples[1:] if w]
+                if not clk and not pw:
+                    return "no sensor samples"
+                return (f"sclk median {statistics.median(clk):.0f} MHz of {len(clk)} samples" if clk else "no clock samples") + \
+                       (f", package power median {statistics.median(pw):.0f} W" if pw else "")
+
+        def b2b(fn, n=args.steps, sensors=None):
+            for _ in range(max(10, args.warmup)):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            if sensors is not None:
+                sensors.__enter__()
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            if sensors is not None:
+                sensors.__exit__()
+            return e0.elapsed_time(e1) * 1e3 / n
+
+        t_settle = time.perf_counter()  # the first loop would otherwise run while the power management still ramps up
+        while (time.perf_counter() - t_settle) * 1e3 < max(args.settle_ms, 500.0):
+            for _ in range(10):
+                gemm()
+            torch.cuda.synchronize()
+
+        ops = 2.0 * M * N * K
+        for name, xs in (("synthetic activations", xd), ("all-zero activations", torch.zeros_like(xd)), ("synthetic activations again", xd)):
+            svdq_quantize_w4a4_act_fuse_lora(xs, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"], fp4=fp4)
+            sens = Sensors()
+            us = b2b(gemm, sensors=sens)
+            print(f"power {args.workload}: W4A4 GEMM kernel, {name}: {us:.1f} us per launch, {ops / us / 1e6:.0f} TOPS ({sens.text()})", flush=True)
+        for dt in (torch.float16, torch.bfloat16, torch.int8):
+            for kind in ("random", "zero"):
+                if dt == torch.int8:
+                    a = torch.randint(-127, 128, (M_pad, K), device=dev, dtype=torch.int8) if kind == "random" else torch.zeros(M_pad, K, device=dev, dtype=torch.int8)
+                    b = torch.randint(-127, 128, (K, N), device=dev, dtype=torch.int8) if kind == "random" else torch.zeros(K, N, device=dev, dtype=torch.int8)
+                    try:
+                        sens = Sensors()
+                        us = b2b(lambda: torch._int_mm(a, b), sensors=sens)
+                    except Exception as exc:  # the library has no such kernel for the shape
+                        print(f"power {args.workload}: vendor int8 GEMM unavailable: {type(exc).__name__}: {exc}", flush=True)
+                        break
+                else:
+                    a = (torch.randn(M_pad, K, device=dev) if kind == "random" else torch.zeros(M_pad, K, device=dev)).to(dt)
+                    b = (torch.randn(N, K, device=dev) if kind == "random" else torch.zeros(N, K, device=dev)).to(dt)
+                    o = torch.empty(M_pad, N, device=dev, dtype=dt)
+                    sens = Sensors()
+                    us = b2b(lambda: torch.matmul(a, b.t(), out=o), sensors=sens)
+                print(f"power {args.workload}: vendor dense GEMM {str(dt).split('.')[-1]} M={M_pad} K={K} N={N}, {kind} operands: {us:.1f} us per launch, "
+                      f"{2.0 * M_pad * N * K / us / 1e6:.0f} T(FL)OPS ({sens.text()})", flush=True)
+        return
     if args.only:
         svdq_quantize_w4a4_act_fuse_lora(xd, output=qx, oscales=asc, lora_down=t["proj_down"], lora_act_out=la, smooth=t["smooth_factor"], fp4=fp4)
         torch.cuda.synchronize()
@@ -332,7 +436,7 @@ def main():
         "roofline": {
             "kernel": (f"gemm_w4a4_kernel<{'true' if args.qkv_rope else 'false'}>" if fp4 else f"g6::gemm6_kernel<{'true' if args.qkv_rope else 'false'}>"),
             "bound": "mfma", "achieved": gemm_tops, "peak": INT8_PEAK_TOPS,
-            "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": PROFILED_GEMM_TRAFFIC_BYTES.get(args.workload),
+            "unit": "TFLOP/s", "frac": gemm_tops / INT8_PEAK_TOPS, "traffic": None if args.qkv_rope else PROFILED_GEMM_TRAFFIC_BYTES.get(args.workload),
             "peak_basis": "dense INT8 MFMA (the metric's peak)" + ("; the NVFP4 kernel issues fp16 MFMA, dense peak 2500" if fp4 else
                           "; the INT4 kernel issues one fp6 MFMA (dense peak 10100) and one small bf16 MFMA per 32x32 tile and k-group"),
         },
