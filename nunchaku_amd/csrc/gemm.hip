@@ -224,9 +224,10 @@ bool acquire_workspace(bool noalloc, int dev, hipStream_t st, size_t zero_bytes,
 // them all, which only pays while compute units would otherwise stand idle.  Below that, a model of the time in us,
 // fitted to launches of 24 ... 216 tiles at K = 3072 and 12288 on 256 compute units: a k-group takes a workgroup 0.55 us
 // while it has its compute unit to itself and 0.95 us when two share one; prologue and epilogue 4.4; a split costs
-// 5.3 + 2.6 per part beyond the first, half as much again when compute units are shared.  Measured, whole / best
-// split: 24 tiles at K = 3072 30.8 / 23.8 (3 parts), 72 tiles 31.0 / 26.9 (3), 96 tiles 31.4 / 28.6 (2), 144 tiles
-// 31.8 / 36.7 (not split); K = 12288: 24 tiles 104.5 / 39.3 (6), 72 tiles 104.8 / 51.4 (3), 144 tiles 105.0 / 75.2 (3).
+// 5.3 + 2.6 per part beyond the first (four parts, whose last one keeps its own sums in registers: 11.5), half as much
+// again when compute units are shared.  Measured, whole / best split: 24 tiles at K = 3072 31.2 / 22.5 (4 parts; 3
+// parts 24.2), 72 tiles 31.3 / 27.3 (3), 96 tiles 31.8 / 31.0 (2; not split), 144 tiles 32.1 / 38.1 (not split);
+// K = 12288: 24 tiles 105.9 / 39.6 (6), 72 tiles 105.6 / 51.7 (3), 144 tiles 106.2 / 78.4 (3).
 int choose_kparts(int ntiles, int kgroups, int ncu) {
     if (ntiles > ncu) return 1;
     int best = 1;
@@ -235,7 +236,7 @@ int choose_kparts(int ntiles, int kgroups, int ncu) {
         const int units = ntiles * k, g = (kgroups + k - 1) / k;
         if (g < 12 || units > 2 * ncu) break;
         const bool shared = units > ncu;
-        const double t = g * (shared ? 0.95 : 0.55) + 4.4 + (5.3 + 2.6 * (k - 1)) * (shared ? 1.5 : 1.0);
+        const double t = g * (shared ? 0.95 : 0.55) + 4.4 + (k == 4 ? 11.5 : 5.3 + 2.6 * (k - 1)) * (shared ? 1.5 : 1.0);
         if (t < (best == 1 ? 0.90 : 0.95) * best_t) {  // a split has to pay clearly; more parts likewise
             best = k;
             best_t = t;

@@ -290,8 +290,8 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
 
     // ---- a tile split along K --------------------------------------------------------------------
     // Every part parks its sums in its slot of the workspace; whoever arrives last adds all parts in
-    // ascending order (its own from memory too, so the result does not depend on who that is) and runs
-    // the epilogue.  Nobody waits for anybody.
+    // ascending order, so the result does not depend on who that is, and runs the epilogue.  Nobody waits for
+    // anybody.
     if (p.kparts > 1) {
         float *slot = p.partials + ((size_t)tile * p.kparts + part) * PARTIAL_SLOT_FLOATS;
         const __amdgpu_buffer_rsrc_t mine = partial_rsrc(slot);
@@ -310,34 +310,78 @@ __global__ void __launch_bounds__(256, 2) gemm6_kernel(Params p) {
         const bool last = *flag == p.kparts - 1;
         if (!last) return;
         if (tid == 0) __hip_atomic_store(p.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        // Four parts (what the launcher chooses for the fewest tiles): the last one keeps its own sums in its registers
+        // and fetches only the others'.  The sum (((0 + s0) + s1) + s2) + s3 is evaluated in exactly that order whoever
+        // is last: the parts before its own are added up first (from zero), then its own joins (a single addition gives
+        // the same result with its operands exchanged), then the parts after it.  Written without branches: a part on
+        // the wrong side of the own contributes +0, which changes nothing because no sum here is ever -0.  (One form
+        // only: with a form per number of parts the compiler carries the 128 accumulators through the alternatives by
+        // way of scratch memory; with two or three parts the general form below is as fast.)
+        if (p.kparts == 4) {
+            constexpr int NOTH = 3;  // the other parts, j-th of them in ascending order: part j + (j >= own)
+            __amdgpu_buffer_rsrc_t r[NOTH];
 #pragma unroll
-        for (int t = 0; t < 8; t++)
+            for (int j = 0; j < NOTH; j++) r[j] = partial_rsrc(p.partials + ((size_t)tile * 4 + j + (j >= part ? 1 : 0)) * PARTIAL_SLOT_FLOATS);
+            // (items of half a 32 x 32 block: 8 accumulators per lane and part; a ring of three, two in flight)
+            float4_t o[3][NOTH][2];
+            auto request = [&](int i) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[t][e] = 0.f;
-        // (two parts at a time, the requests of the next eighth of the tile in flight while this one is added;
-        // every element still adds its parts in ascending order)
-        for (int pt0 = 0; pt0 < p.kparts; pt0 += 2) {
-            const bool two = pt0 + 1 < p.kparts;
-            const __amdgpu_buffer_rsrc_t r0 = partial_rsrc(p.partials + ((size_t)tile * p.kparts + pt0) * PARTIAL_SLOT_FLOATS);
-            const __amdgpu_buffer_rsrc_t r1 = partial_rsrc(p.partials + ((size_t)tile * p.kparts + (two ? pt0 + 1 : pt0)) * PARTIAL_SLOT_FLOATS);
-            float4_t o[2][2][4];
-            auto request = [&](int t, int b) {
+                for (int j = 0; j < NOTH; j++)
 #pragma unroll
-                for (int q = 0; q < 4; q++) o[b][0][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r0, ((t * 4 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
-                if (two) {
-#pragma unroll
-                    for (int q = 0; q < 4; q++) o[b][1][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r1, ((t * 4 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
-                }
+                    for (int q = 0; q < 2; q++)
+                        o[i % 3][j][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r[j], ((i * 2 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
             };
-            request(0, 0);
+            request(0);
+            request(1);
 #pragma unroll
-            for (int t = 0; t < 8; t++) {
-                if (t + 1 < 8) request(t + 1, (t + 1) & 1);
+            for (int i = 0; i < 16; i++) {
+                if (i + 2 < 16) request(i + 2);
+                const int t = i >> 1, e0 = (i & 1) * 8;
+                float before[8];
 #pragma unroll
-                for (int e = 0; e < 16; e++) acc[t][e] += o[t & 1][0][e / 4][e % 4];
-                if (two) {
+                for (int e = 0; e < 8; e++) before[e] = 0.f;
 #pragma unroll
-                    for (int e = 0; e < 16; e++) acc[t][e] += o[t & 1][1][e / 4][e % 4];
+                for (int j = 0; j < NOTH; j++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) before[e] += j < part ? o[i % 3][j][e / 4][e % 4] : 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[t][e0 + e] = before[e] + acc[t][e0 + e];
+#pragma unroll
+                for (int j = 0; j < NOTH; j++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[t][e0 + e] += j >= part ? o[i % 3][j][e / 4][e % 4] : 0.f;
+            }
+        } else {
+            // any other number of parts: all of them from memory, the own included (a running sum of the parts before
+            // the own would need a second set of accumulators beyond four parts), two parts at a time, the requests of the next eighth of the tile in
+            // flight while one is added; every element still adds its parts in ascending order
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[t][e] = 0.f;
+            for (int pt0 = 0; pt0 < p.kparts; pt0 += 2) {
+                const bool two = pt0 + 1 < p.kparts;
+                const __amdgpu_buffer_rsrc_t r0 = partial_rsrc(p.partials + ((size_t)tile * p.kparts + pt0) * PARTIAL_SLOT_FLOATS);
+                const __amdgpu_buffer_rsrc_t r1 = partial_rsrc(p.partials + ((size_t)tile * p.kparts + (two ? pt0 + 1 : pt0)) * PARTIAL_SLOT_FLOATS);
+                float4_t o[2][2][4];
+                auto request = [&](int t, int b) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) o[b][0][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r0, ((t * 4 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
+                    if (two) {
+#pragma unroll
+                        for (int q = 0; q < 4; q++) o[b][1][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r1, ((t * 4 + q) * 256 + tid) * 16, 0, PARTIAL_SC0_SC1));
+                    }
+                };
+                request(0, 0);
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    if (t + 1 < 8) request(t + 1, (t + 1) & 1);
+#pragma unroll
+                    for (int e = 0; e < 16; e++) acc[t][e] += o[t & 1][0][e / 4][e % 4];
+                    if (two) {
+#pragma unroll
+                        for (int e = 0; e < 16; e++) acc[t][e] += o[t & 1][1][e / 4][e % 4];
+                    }
                 }
             }
         }

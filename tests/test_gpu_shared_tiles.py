@@ -34,7 +34,7 @@ def _inputs(M_pad, K, R, seed):
 )
 def test_split_tiles_match_whole_tiles(dev, M, K, N, R, k_split, monkeypatch):
     """k_split None: the library's own choice for a shape with few tiles (M = 256, K = N = 3072: 24 tiles,
-    3 parts each; M = 512, K = 12288, N = 512: 8 tiles, 8 parts each); 10 parts of K = 640: one k-group each; N = 384 and 1280: a ragged last column block."""
+    4 parts each; M = 512, K = 12288, N = 512: 8 tiles, 8 parts each); 10 parts of K = 640: one k-group each; N = 384 and 1280: a ragged last column block."""
     from nunchaku_amd import packing
     from nunchaku_amd.ops import gemm as gemm_mod
 
