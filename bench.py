@@ -15,8 +15,11 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import statistics
+import subprocess
 import sys
+import threading
 import time
 from pathlib import Path
 
@@ -51,6 +54,41 @@ PROFILED_GEMM_FETCH_WRITE_KIB = {
 }
 PROFILED_GEMM_TRAFFIC_BYTES = {w: (FETCH_SCALE * f + WRITE_SCALE * wr) * 1024 for w, (f, wr) in PROFILED_GEMM_FETCH_WRITE_KIB.items()}
 HBM_PEAK_GBS = 8000.0
+
+
+class Sensors:
+    """Shader clock and package power as `rocm-smi` reports them, sampled by a thread while a timed loop runs."""
+
+    def __init__(self):
+        self.samples, self.stop = [], threading.Event()
+
+    def _run(self):
+        while not self.stop.is_set():
+            try:
+                txt = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--json"], capture_output=True, text=True, timeout=10).stdout
+                card = next(iter(json.loads(txt).values()))
+                clk = [float(re.search(r"(\d+)\s*Mhz", v, re.I).group(1)) for k, v in card.items() if k.lower().startswith("sclk") and re.search(r"(\d+)\s*Mhz", str(v), re.I)]
+                pw = [float(v) for k, v in card.items() if "power" in k.lower() and re.fullmatch(r"[\d.]+", str(v).strip())]
+                self.samples.append((clk[0] if clk else None, pw[0] if pw else None))
+            except Exception:  # no tool, no permission, another output format: the timings stand without it
+                return
+
+    def __enter__(self):
+        self.thread = threading.Thread(target=self._run, daemon=True)
+        self.thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self.stop.set()
+        self.thread.join(timeout=15)
+
+    def text(self):
+        clk = [c for c, _ in self.samples[1:] if c]  # (the first sample may predate the loop)
+        pw = [w for _, w in self.samples[1:] if w]
+        if not clk and not pw:
+            return "no sensor samples"
+        return (f"sclk median {statistics.median(clk):.0f} MHz of {len(clk)} samples" if clk else "no clock samples") + \
+               (f", package power median {statistics.median(pw):.0f} W" if pw else "")
 
 
 def cpu_baseline(layer, x, rows: int, iters: int = 20):
@@ -252,44 +290,6 @@ def main():
         gemm()
 
     if args.only == "power":
-        import re
-        import subprocess
-        import threading
-
-        class Sensors:
-            """Shader clock and package power as `rocm-smi` reports them, sampled by a thread while a timed loop runs."""
-
-            def __init__(self):
-                self.samples, self.stop = [], threading.Event()
-
-            def _run(self):
-                while not self.stop.is_set():
-                    try:
-                        txt = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--json"], capture_output=True, text=True, timeout=10).stdout
-                        card = next(iter(json.loads(txt).values()))
-                        clk = [float(re.search(r"(\d+)\s*Mhz", v, re.I).group(1)) for k, v in card.items() if k.lower().startswith("sclk") and re.search(r"(\d+)\s*Mhz", str(v), re.I)]
-                        pw = [float(v) for k, v in card.items() if "power" in k.lower() and re.fullmatch(r"[\d.]+", str(v).strip())]
-                        self.samples.append((clk[0] if clk else None, pw[0] if pw else None))
-                    except Exception:  # no tool, no permission, another output format: the timings stand without it
-                        return
-
-            def __enter__(self):
-                self.thread = threading.Thread(target=self._run, daemon=True)
-                self.thread.start()
-                return self
-
-            def __exit__(self, *exc):
-                self.stop.set()
-                self.thread.join(timeout=15)
-
-            def text(self):
-                clk = [c for c, _ in self.samples[1:] if c]  # (the first sample may predate the loop)
-                pw = [w for _, w in self.samples[1:] if w]
-                if not clk and not pw:
-                    return "no sensor samples"
-                return (f"sclk median {statistics.median(clk):.0f} MHz of {len(clk)} samples" if clk else "no clock samples") + \
-                       (f", package power median {statistics.median(pw):.0f} W" if pw else "")
-
         def b2b(fn, n=args.steps, sensors=None):
             for _ in range(max(10, args.warmup)):
                 fn()
@@ -409,6 +409,24 @@ def main():
     torch.cuda.synchronize()
     tg_b2b_us = g0.elapsed_time(g1) * 1e3 / args.steps
     tg_step_us = ms_per_step_events * 1e3 - tq_b2b_us
+    # The shader clock while the step runs (outside the timed region: about a second of the same steps with a thread
+    # reading `rocm-smi`).  The GEMM is bound by the chip's power limit: the clock the power management grants on these
+    # operands, against the 2400 MHz that the published peaks assume, is part of what `roofline.frac` measures.  Not
+    # under a profiler, whose preloaded tool would load into the child processes too.
+    clock = None
+    profiled = any("rocprof" in os.environ.get(k, "").lower() for k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB", "ROCPROFILER_LIBRARY_PATH"))
+    if not profiled:
+        sens = Sensors()
+        with sens:
+            t_clk = time.perf_counter()
+            while time.perf_counter() - t_clk < 1.0:
+                for _ in range(20):
+                    step()
+                torch.cuda.synchronize()
+        clk = [c for c, _ in sens.samples[1:] if c]
+        if clk:
+            clock = {"sclk_mhz_median_during_steps": statistics.median(clk), "samples": len(clk), "published_peak_clock_mhz": 2400,
+                     "source": "rocm-smi --showclocks, sampled for one second of the same steps after the timed region"}
 
     ops_layer = 2.0 * M * N * K + 2.0 * M * R * (K + N)
     ops_gemm = 2.0 * M * N * K + 2.0 * M * R * N
@@ -424,6 +442,7 @@ def main():
                                + (" + RMS norm and rotary embedding on q, k in the GEMM epilogue" if args.qkv_rope else ""),
                    "M": M, "K": K, "N": N, "rank": R},
         "pct_of_int8_mfma_peak": 100.0 * value / INT8_PEAK_TOPS,
+        "clock": clock,
         "us_per_layer": ms_per_step * 1e3,
         "us_per_layer_events": ms_per_step_events * 1e3,
         "kernels": {
