@@ -132,6 +132,31 @@ def test_scanner_finds_a_carry_kept_across_an_asm_add():
     assert scc_live_across_asm(good) == []
 
 
+def test_the_build_before_the_clobbers_were_declared_kept_flags_across_the_copies():
+    """The sources as they were before the commit that declared what the copy statements overwrite (``07f9e0a``),
+    taken from the repository's history and compiled with today's flags: the scanner finds condition-code values kept
+    alive across copy statements there (the carry of a 64-bit source pointer among them) and none in today's sources
+    (``test_no_condition_code_kept_across_inline_asm``).  Skipped where the history is not at hand."""
+    root = CSRC.parents[1]
+    old = "07f9e0a^"
+    probe = subprocess.run(["git", "-C", str(root), "cat-file", "-e", f"{old}:nunchaku_amd/csrc/gemm6_kernel.h"], capture_output=True)
+    if probe.returncode != 0:
+        pytest.skip("no git history with the earlier sources here")
+    flags = [f for f in nv.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    with tempfile.TemporaryDirectory(prefix="svdq_guard_old_") as tmp:
+        tar = subprocess.run(["git", "-C", str(root), "archive", old, "nunchaku_amd/csrc", "include"], capture_output=True)
+        assert tar.returncode == 0, tar.stderr[-500:]
+        subprocess.run(["tar", "-x", "-C", tmp], input=tar.stdout, check=True)
+        out = Path(tmp) / "old.s"
+        res = subprocess.run(["/opt/rocm/bin/hipcc", *flags, "-DSVDQ_VARIANT=0", "-S", "--cuda-device-only",
+                              str(Path(tmp) / "nunchaku_amd/csrc/gemm6_variant.hip"), "-o", str(out)], capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr[-3000:]
+        bad = scc_live_across_asm(out.read_text().splitlines())
+    print(bad)
+    assert bad, "the earlier build shows no condition code kept across an inline-asm statement"
+    assert any(text.startswith("s_addc_u32") for _, text in bad), bad  # a lost carry: the source pointer of a copy, 4 GiB too low
+
+
 @pytest.fixture(scope="module")
 def compiled():
     units = [("gemm6_variant.hip", 0), ("gemm6_variant.hip", 1), ("gemm_variant.hip", 4), ("gemm_variant.hip", 5)]
