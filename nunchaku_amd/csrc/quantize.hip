@@ -69,7 +69,7 @@ template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU,
 __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams p) {
     // smoothing factors [K] during the walk; then, chunks split: [NW waves][MT][RT][64][4] partial projections;
     // rows split: behind the factors two buffers of [4 steps][RT][64 lanes] x 16 bytes of proj_down
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];  // (the alignment lets the factors be read 16 bytes at a time)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, q = lane >> 4;
@@ -171,19 +171,25 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
     auto process = [&](int c, u32x4_t (&xin)[MT][XL], u32x4_t (&x_ahead)[MT][XL]) {
         const int kbase = 128 * c + 32 * q;
         // ---- from the load layout to the operand layout: lane (r, q) gets the XL pieces XL * q + i of row r.
-        // Row-major in LDS with the pieces of row r rotated by r: the 16 lanes of a write (one row, 16 pieces)
-        // and the 16 lanes of a read (16 rows, one piece) then both hit 16 different bank groups.  The area is
-        // private to the wave, whose LDS operations complete in order.
+        // Row-major in LDS with the pieces of row r rotated by rot(r).  A 16-byte write is served eight consecutive
+        // lanes at a time (one row, consecutive pieces: any rotation will do).  A 16-byte read is served 16 lanes at
+        // a time, and not consecutive ones: lanes 0-3, 12-15 and 20-27 together, then 4-11, 16-19 and 28-31 (measured
+        // pair by pair; the same in the upper half-wave), that is rows {0-3, 12-15} of one q with rows {4-11} of
+        // the next.  Their pieces are XL apart, so the rotation must send both row sets to one set of eight 16-byte
+        // bank groups that, moved by XL, gives the other eight: r with bit 2 cleared for XL = 4, and for XL = 8 the
+        // low two bits of r with bits 2 and 3 both set to bit 3 (with rot(r) = r every such read took two turns).
+        // The area is private to the wave, whose LDS operations complete in order.
+        auto rot = [](int row) { return XL == 4 ? (row & 11) : ((row & 3) | ((row & 8) ? 12 : 0)); };
         u32x4_t xraw[MT][XL];
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
             for (int i = 0; i < XL; i++) {
                 const int row = RPI * i + lane / PPR, piece = lane % PPR;
-                *(u32x4_t *)(tr + row * (PPR * 16) + ((piece + row) % PPR) * 16) = xin[mt][i];
+                *(u32x4_t *)(tr + row * (PPR * 16) + ((piece + rot(row)) % PPR) * 16) = xin[mt][i];
             }
 #pragma unroll
-            for (int i = 0; i < XL; i++) xraw[mt][i] = *(const u32x4_t *)(tr + r * (PPR * 16) + ((XL * q + i + r) % PPR) * 16);
+            for (int i = 0; i < XL; i++) xraw[mt][i] = *(const u32x4_t *)(tr + r * (PPR * 16) + ((XL * q + i + rot(r)) % PPR) * 16);
         }
         // ---- requests first: the low-rank operands of this chunk (all four steps when they fit the
         // registers), then the activations DEPTH chunks ahead.  In this order a wait for the operands
