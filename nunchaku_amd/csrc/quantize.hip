@@ -37,7 +37,6 @@ struct QuantParams {
     const float *smooth_rcp; // [K] or null
     int M, M_pad, K, R;
     int rt_base;             // first 16-rank tile of the projection this launch computes (ranks above 128 take several launches)
-    int rows_per_wg;         // rows a workgroup owns when its waves split the chunks: 16 MT, or fewer (see PART)
 };
 
 constexpr uint32_t RSRC_WORD3 = 0x00020000;  // raw buffer, 32-bit data format
@@ -60,12 +59,7 @@ constexpr uint32_t RSRC_WORD3 = 0x00020000;  // raw buffer, 32-bit data format
 // Ranks above 16 RT_MAX: a launch projects onto the rank tiles [rt_base, rt_base + RT_MAX) only (its accumulators
 // live in registers), so the operator launches the kernel once per window of 128 ranks; the launches after the
 // first (QUANT false) read x again, which the caches still hold, and neither quantize nor store codes.
-//
-// PART (balance): a workgroup owns p.rows_per_wg < 16 MT rows, so that the row count divides evenly among the compute
-// units where 16-row blocks do not (4608 rows on 256 compute units: 18 rows each instead of 16 for most and 32 for
-// some, which finish last).  The row slots beyond the owned rows belong to the next workgroup: they read as zero
-// through the buffer descriptor, cost no memory traffic, and nothing is stored for them.
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS, bool QUANT = true, bool PART = false>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS, bool QUANT = true>
 __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams p) {
     // smoothing factors [K] during the walk; then, chunks split: [NW waves][MT][RT][64][4] partial projections;
     // rows split: behind the factors two buffers of [4 steps][RT][64 lanes] x 16 bytes of proj_down
@@ -73,9 +67,8 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, q = lane >> 4;
-    const int row0 = ROWS ? (blockIdx.x * NW + wave) * (16 * MT) : blockIdx.x * (PART ? p.rows_per_wg : 16 * MT);
-    int row_end = row0 + (PART ? p.rows_per_wg : 16 * MT);  // the rows this workgroup (ROWS: wave) writes are [row0, row_end)
-    if (PART && row_end > p.M_pad) row_end = p.M_pad;
+    const int row0 = ROWS ? (blockIdx.x * NW + wave) * (16 * MT) : blockIdx.x * (16 * MT);
+    const int row_end = row0 + 16 * MT;  // the rows this workgroup (ROWS: wave) writes are [row0, row_end)
     const int kgroups = p.K / 64;
     const int RT_all = p.R / 16;                                                         // rank tiles of proj_down and lora_out
     const int RT = RT_all - p.rt_base < RT_MAX ? RT_all - p.rt_base : RT_MAX;            // rank tiles of this launch
@@ -275,14 +268,12 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
                 u32x2_t hi;
                 float s;
                 quantize_int4_half_group_e2m3<false>(y, 16, lo, hi, s);
-                if (!PART || row < row_end) {
-                    // (both lanes of a group hold the same scale and store it: no branch)
-                    ((uint16_t *)p.oscales)[(size_t)(2 * c + (q >> 1)) * p.M_pad + row] = (uint16_t)f32_to_bf16_bits(s);
-                    uint8_t *frag = p.act + (((size_t)(row / ACT_BLOCK_ROWS) * kgroups + (2 * c + (q >> 1))) * 4 + (row % ACT_BLOCK_ROWS) / 32) * FRAG_BYTES;
-                    const int slot = (row % 32) + 32 * (q & 1);
-                    *(u32x4_t *)(frag + slot * 16) = lo;
-                    *(u32x2_t *)(frag + 1024 + slot * 8) = hi;
-                }
+                // (both lanes of a group hold the same scale and store it: no branch)
+                ((uint16_t *)p.oscales)[(size_t)(2 * c + (q >> 1)) * p.M_pad + row] = (uint16_t)f32_to_bf16_bits(s);
+                uint8_t *frag = p.act + (((size_t)(row / ACT_BLOCK_ROWS) * kgroups + (2 * c + (q >> 1))) * 4 + (row % ACT_BLOCK_ROWS) / 32) * FRAG_BYTES;
+                const int slot = (row % 32) + 32 * (q & 1);
+                *(u32x4_t *)(frag + slot * 16) = lo;
+                *(u32x2_t *)(frag + 1024 + slot * 8) = hi;
             } else {
                 const size_t tile = (size_t)(row / 32) * kgroups + (2 * c + (q >> 1));
                 uint8_t *dst = p.act + tile * TILE_BYTES + (row % 32) * 32 + 16 * (q & 1);
@@ -290,11 +281,9 @@ __global__ void __launch_bounds__(64 * NW) quantize_fuse_lora_kernel(QuantParams
                 uint32_t sc[2];
                 quantize_nvfp4_two_groups(y, words, sc);
                 // NVFP4 scales: [K/64][M_pad][4] -- the four 16-groups of a 64-group side by side
-                if (!PART || row < row_end) {
-                    uint16_t *os = (uint16_t *)p.oscales;
-                    os[((size_t)(2 * c + (q >> 1)) * p.M_pad + row) * 2 + (q & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
-                    *(u32x4_t *)dst = words;
-                }
+                uint16_t *os = (uint16_t *)p.oscales;
+                os[((size_t)(2 * c + (q >> 1)) * p.M_pad + row) * 2 + (q & 1)] = (uint16_t)(sc[0] | (sc[1] << 8));
+                *(u32x4_t *)dst = words;
             }
         }
 
@@ -360,34 +349,34 @@ walked:
             float sum = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; w++) sum += lds[(((w * MT + mt) * RT + rt) * 64 + src_lane) * 4 + i];
-            if (!PART || row0 + row < row_end) p.lora_out[(size_t)(row0 + row) * p.R + 16 * p.rt_base + rank] = sum;
+            p.lora_out[(size_t)(row0 + row) * p.R + 16 * p.rt_base + rank] = sum;
         }
     }
 }
 
 constexpr size_t SMOOTH_LDS_MAX = 64 * 1024;  // two workgroups of a compute unit must fit side by side
 
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS = false, bool QUANT = true, bool PART = false>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, int SMOOTH, bool GLU, bool ROWS = false, bool QUANT = true>
 int launch_as(const QuantParams &p, hipStream_t stream) {
     const int rt_launch = p.R / 16 - p.rt_base < RT_MAX ? p.R / 16 - p.rt_base : RT_MAX;
     size_t smem = (size_t)NW * MT * rt_launch * 64 * 4 * sizeof(float);
     if (SMOOTH == 1 && (size_t)p.K * 4 > smem) smem = (size_t)p.K * 4;
     if (ROWS) smem = (SMOOTH == 1 ? (size_t)p.K * 4 : 0) + 2 * (size_t)(p.R / 16) * 4096;
-    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH, GLU, ROWS, QUANT, PART>;
+    auto kern = quantize_fuse_lora_kernel<NW, MT, RT_MAX, DEPTH, FP4, SMOOTH, GLU, ROWS, QUANT>;
     if (smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return fail(SVDQ_ELAUNCH, "quantize: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
     }
-    const int rows_per_wg = PART ? p.rows_per_wg : 16 * MT * (ROWS ? NW : 1);
+    const int rows_per_wg = 16 * MT * (ROWS ? NW : 1);
     SVDQ_LAUNCH(kern, dim3((p.M_pad + rows_per_wg - 1) / rows_per_wg), dim3(64 * NW), smem, stream, p);
     return check_launch("quantize_w4a4_act_fuse_lora");
 }
 
-template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, bool GLU, bool ROWS = false, bool PART = false>
+template <int NW, int MT, int RT_MAX, int DEPTH, bool FP4, bool GLU, bool ROWS = false>
 int launch(const QuantParams &p, hipStream_t stream) {
-    if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0, GLU, ROWS, true, PART>(p, stream);
-    if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1, GLU, ROWS, true, PART>(p, stream);
-    return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2, GLU, ROWS, true, PART>(p, stream);
+    if (!p.smooth_rcp) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 0, GLU, ROWS, true>(p, stream);
+    if ((size_t)p.K * 4 <= SMOOTH_LDS_MAX) return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 1, GLU, ROWS, true>(p, stream);
+    return launch_as<NW, MT, RT_MAX, DEPTH, FP4, 2, GLU, ROWS, true>(p, stream);
 }
 
 // the rank tiles from 8 on, 8 per launch: projection only (no smoothing factors, no codes, either precision)
@@ -403,9 +392,8 @@ int project_further(const QuantParams &p0, hipStream_t stream) {
 
 template <bool FP4, bool GLU>
 int dispatch(const QuantParams &p, hipStream_t stream) {
-    // Rows per workgroup: 16 while that gives the chip enough workgroups, 32 to amortise the proj_down
-    // reads at high rank.  Four waves of up to 256 registers: two workgroups fit a compute unit, so that a
-    // workgroup count a little above the number of compute units does not cost a second round.
+    // Rows and waves per workgroup by shape and rank, from measurements (below).  At ranks above 32: four waves, 32 rows
+    // to amortise the proj_down reads (two such workgroups fit a compute unit).
     const int RT = p.R / 16;
     // (with GLU a chunk in flight is twice the registers: one chunk ahead, 16 rows)
     if (GLU) {
@@ -422,20 +410,20 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         if (RT > 2 && RT <= 4 && p.M_pad >= 256 * 64) return launch<4, 1, 4, 1, FP4, false, true>(p, stream);
         // Up to one 16-row workgroup per compute unit (256 of them) the walk over K is what takes the time: eight waves
         // split it (M = 256 ... 4096 at K = 3072: 7.9 ... 10.1 us against 9.0 ... 11.3 with four; K = 12288, M = 256:
-        // 19.6 against 25.5).  Beyond that two four-wave workgroups share a compute unit better (M = 4608: 14.4 against 16.2).
+        // 19.6 against 25.5).
         int dev = 0;
         const int ncu = hipGetDevice(&dev) == hipSuccess && compute_units(dev) > 0 ? compute_units(dev) : 256;
         if (RT <= 2 && p.M_pad <= 16 * ncu) return launch<8, 1, 2, 1, FP4, false>(p, stream);
-        if (RT <= 2 && p.M_pad < 32 * ncu) {
-            // Between one and two 16-row blocks per compute unit, whole blocks leave some compute units with two and
-            // most with one, and those with two finish last (M = 4608 on 256 compute units: 13.5 us against 10.3 at
-            // M = 4096).  Every workgroup takes ceil(M_pad / ncu) rows instead, two row tiles of which the second is
-            // partly filled: the same rows on every compute unit.
-            QuantParams q = p;
-            q.rows_per_wg = (p.M_pad + ncu - 1) / ncu;
-            return launch<8, 2, 2, 1, FP4, false, false, true>(q, stream);
-        }
-        if (RT <= 2) return launch<4, 2, 2, 1, FP4, false>(p, stream);
+        // Beyond that, at ranks up to 32 (measured at K = 3072 unless noted, on 256 compute units):
+        //   up to two 16-row blocks per compute unit, and long rows at any M: eight waves on 32 rows, fewer workgroups
+        //   than compute units included (M = 4608: 11.5 us against 12.6 for one workgroup per compute unit with equal
+        //   shares of the rows, whose partly filled second block costs its full arithmetic, and 13.3 for 288 workgroups of
+        //   16 rows; K = 12288: 31.9 against 33.5 and 40.0);
+        //   more rows than that with short rows: many small workgroups, four waves on 16 rows with two chunks requested
+        //   ahead (M = 12288: 22.0 us against 25.3; K = 4096: 31.4 against 40.8; M = 18432: 31.5 against 35.6; equal from
+        //   M = 36864 on and at K = 6144 from M = 18432 on).
+        if (RT <= 2 && (p.M_pad <= 32 * ncu || p.K > 6144 || p.M_pad >= 128 * ncu)) return launch<8, 2, 2, 1, FP4, false>(p, stream);
+        if (RT <= 2) return launch<4, 1, 2, 2, FP4, false>(p, stream);
         if (RT <= 4) return launch<4, 2, 4, 1, FP4, false>(p, stream);
         if (RT <= 8) return launch<4, 2, 8, 1, FP4, false>(p, stream);
         // ranks above 128: the first 128 with the codes, the rest in further launches over the same rows
@@ -467,7 +455,6 @@ extern "C" int svdq_quantize_w4a4_act_fuse_lora(const svdq_quantize_args *a, voi
     p.smooth_rcp = a->smooth_rcp;
     p.M = (int)a->M; p.M_pad = (int)a->M_pad; p.K = (int)a->K; p.R = (int)a->R;
     p.rt_base = 0;
-    p.rows_per_wg = 0;
     hipStream_t s = (hipStream_t)stream;
     if (a->fuse_glu) return a->fp4 ? dispatch<true, true>(p, s) : dispatch<false, true>(p, s);
     return a->fp4 ? dispatch<true, false>(p, s) : dispatch<false, false>(p, s);
