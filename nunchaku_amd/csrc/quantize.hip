@@ -380,11 +380,11 @@ int launch(const QuantParams &p, hipStream_t stream) {
 }
 
 // the rank tiles from 8 on, 8 per launch: projection only (no smoothing factors, no codes, either precision)
-template <int NW, int MT, bool GLU>
+template <int NW, int MT, int DEPTH, bool GLU>
 int project_further(const QuantParams &p0, hipStream_t stream) {
     QuantParams p = p0;
     for (p.rt_base = 8; p.rt_base < p.R / 16; p.rt_base += 8) {
-        const int rc = launch_as<NW, MT, 8, 1, false, 0, GLU, false, false>(p, stream);
+        const int rc = launch_as<NW, MT, 8, DEPTH, false, 0, GLU, false, false>(p, stream);
         if (rc != SVDQ_OK) return rc;
     }
     return SVDQ_OK;
@@ -392,8 +392,7 @@ int project_further(const QuantParams &p0, hipStream_t stream) {
 
 template <bool FP4, bool GLU>
 int dispatch(const QuantParams &p, hipStream_t stream) {
-    // Rows and waves per workgroup by shape and rank, from measurements (below).  At ranks above 32: four waves, 32 rows
-    // to amortise the proj_down reads (two such workgroups fit a compute unit).
+    // Rows and waves per workgroup by shape and rank, from measurements (below).
     const int RT = p.R / 16;
     // (with GLU a chunk in flight is twice the registers: one chunk ahead, 16 rows)
     if (GLU) {
@@ -401,7 +400,7 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         if (RT <= 4) return launch<4, 1, 4, 1, FP4, true>(p, stream);
         if (RT <= 8) return launch<4, 1, 8, 1, FP4, true>(p, stream);
         const int rc = launch<4, 1, 8, 1, FP4, true>(p, stream);
-        return rc != SVDQ_OK ? rc : project_further<4, 1, true>(p, stream);
+        return rc != SVDQ_OK ? rc : project_further<4, 1, 1, true>(p, stream);
     } else {
         // High ranks with enough rows to give every compute unit work: the waves split the rows and share each
         // chunk of proj_down through LDS (M = 18432, K = 3072: rank 128 68 us against 122, rank 64 51 against 71;
@@ -424,11 +423,20 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         //   M = 36864 on and at K = 6144 from M = 18432 on).
         if (RT <= 2 && (p.M_pad <= 32 * ncu || p.K > 6144 || p.M_pad >= 128 * ncu)) return launch<8, 2, 2, 1, FP4, false>(p, stream);
         if (RT <= 2) return launch<4, 1, 2, 2, FP4, false>(p, stream);
-        if (RT <= 4) return launch<4, 2, 4, 1, FP4, false>(p, stream);
-        if (RT <= 8) return launch<4, 2, 8, 1, FP4, false>(p, stream);
+        // Ranks 48 ... 128 below the row counts of the rows-split form: eight waves on 32 rows (M = 4608, K = 3072: rank
+        // 128 28.8 us, rank 64 16.0; four waves on the same rows 44.8 and 22.5; K = 12288, rank 128: 97 against 167);
+        // with few rows (up to 8 per compute unit) many small workgroups with two chunks ahead (M = 2048, rank 128: 18.9
+        // against 25.6; M = 256: 18.2 against 18.6).
+        const bool few_rows = p.M_pad <= 8 * ncu;
+        if (RT <= 4) return few_rows ? launch<4, 1, 4, 2, FP4, false>(p, stream) : launch<8, 2, 4, 1, FP4, false>(p, stream);
+        if (RT <= 8) return few_rows ? launch<4, 1, 8, 2, FP4, false>(p, stream) : launch<8, 2, 8, 1, FP4, false>(p, stream);
         // ranks above 128: the first 128 with the codes, the rest in further launches over the same rows
-        const int rc = launch<4, 2, 8, 1, FP4, false>(p, stream);
-        return rc != SVDQ_OK ? rc : project_further<4, 2, false>(p, stream);
+        if (few_rows) {
+            const int rc = launch<4, 1, 8, 2, FP4, false>(p, stream);
+            return rc != SVDQ_OK ? rc : project_further<4, 1, 2, false>(p, stream);
+        }
+        const int rc = launch<8, 2, 8, 1, FP4, false>(p, stream);
+        return rc != SVDQ_OK ? rc : project_further<8, 2, 1, false>(p, stream);
     }
 }
 
