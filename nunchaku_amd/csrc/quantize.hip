@@ -421,7 +421,9 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         //   more rows than that with short rows: many small workgroups, four waves on 16 rows with two chunks requested
         //   ahead (M = 12288: 22.0 us against 25.3; K = 4096: 31.4 against 40.8; M = 18432: 31.5 against 35.6; equal from
         //   M = 36864 on and at K = 6144 from M = 18432 on).
-        if (RT <= 2 && (p.M_pad <= 32 * ncu || p.K > 6144 || p.M_pad >= 128 * ncu)) return launch<8, 2, 2, 1, FP4, false>(p, stream);
+        //   (NVFP4, whose quantizer is the heavier one, is better off with the small workgroups from 16 rows per compute
+        //   unit on while the rows are short: M = 4608: 12.5 us against 13.4, M = 8192: 15.6 against 16.4)
+        if (RT <= 2 && (p.K > 6144 || p.M_pad >= 128 * ncu || (!FP4 && p.M_pad <= 32 * ncu))) return launch<8, 2, 2, 1, FP4, false>(p, stream);
         if (RT <= 2) return launch<4, 1, 2, 2, FP4, false>(p, stream);
         // Ranks 48 ... 128 below the row counts of the rows-split form: eight waves on 32 rows (M = 4608, K = 3072: rank
         // 128 28.8 us, rank 64 16.0; four waves on the same rows 44.8 and 22.5; K = 12288, rank 128: 97 against 167);
@@ -429,7 +431,9 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         // against 25.6; M = 256: 18.2 against 18.6).
         const bool few_rows = p.M_pad <= 8 * ncu;
         if (RT <= 4) return few_rows ? launch<4, 1, 4, 2, FP4, false>(p, stream) : launch<8, 2, 4, 1, FP4, false>(p, stream);
-        if (RT <= 8) return few_rows ? launch<4, 1, 8, 2, FP4, false>(p, stream) : launch<8, 2, 8, 1, FP4, false>(p, stream);
+        // (NVFP4 at ranks 80 ... 128: the small workgroups at any row count, M = 4608: 29.7 us against 36.0, M = 12288: 57.7
+        // against 71.1, K = 6144: 55.2 against 63.3; at rank 64 the large ones as for INT4, 16.5 against 25.1)
+        if (RT <= 8) return few_rows || FP4 ? launch<4, 1, 8, 2, FP4, false>(p, stream) : launch<8, 2, 8, 1, FP4, false>(p, stream);
         // ranks above 128: the first 128 with the codes, the rest in further launches over the same rows
         if (few_rows) {
             const int rc = launch<4, 1, 8, 2, FP4, false>(p, stream);
