@@ -402,16 +402,17 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         const int rc = launch<4, 1, 8, 1, FP4, true>(p, stream);
         return rc != SVDQ_OK ? rc : project_further<4, 1, 1, true>(p, stream);
     } else {
-        // High ranks with enough rows to give every compute unit work: the waves split the rows and share each
-        // chunk of proj_down through LDS (M = 18432, K = 3072: rank 128 68 us against 122, rank 64 51 against 71;
-        // at M = 4608 the few large workgroups lose: 65 against 42).
-        if (RT > 4 && RT <= 8 && p.M_pad >= 128 * 128) return launch<4, 2, 8, 1, FP4, false, true>(p, stream);
-        if (RT > 2 && RT <= 4 && p.M_pad >= 256 * 64) return launch<4, 1, 4, 1, FP4, false, true>(p, stream);
+        int dev = 0;
+        const int ncu = hipGetDevice(&dev) == hipSuccess && compute_units(dev) > 0 ? compute_units(dev) : 256;
+        // High ranks with many rows: the waves split the rows (eight waves, 128 rows per workgroup) and share each chunk
+        // of proj_down through LDS.  Ranks 80 ... 128, K = 3072: M = 18432 52.4 us (four waves on 32 rows each: 61.8; the
+        // chunk-split forms 87 and more), M = 12288 51.3 against 58.3; below 32 rows per compute unit the chunk-split
+        // form wins (M = 8192: 33.2 against 51.0).  Ranks 48 ... 64: M = 18432 41.0 against 50.7.
+        if (RT > 4 && RT <= 8 && (FP4 ? p.M_pad >= 128 * 128 : p.M_pad > 32 * ncu)) return launch<8, 1, 8, 1, FP4, false, true>(p, stream);
+        if (RT > 2 && RT <= 4 && p.M_pad >= 256 * 64) return launch<8, 1, 4, 1, FP4, false, true>(p, stream);
         // Up to one 16-row workgroup per compute unit (256 of them) the walk over K is what takes the time: eight waves
         // split it (M = 256 ... 4096 at K = 3072: 7.9 ... 10.1 us against 9.0 ... 11.3 with four; K = 12288, M = 256:
         // 19.6 against 25.5).
-        int dev = 0;
-        const int ncu = hipGetDevice(&dev) == hipSuccess && compute_units(dev) > 0 ? compute_units(dev) : 256;
         if (RT <= 2 && p.M_pad <= 16 * ncu) return launch<8, 1, 2, 1, FP4, false>(p, stream);
         // Beyond that, at ranks up to 32 (measured at K = 3072 unless noted, on 256 compute units):
         //   up to two 16-row blocks per compute unit, and long rows at any M: eight waves on 32 rows, fewer workgroups
