@@ -212,6 +212,23 @@ def test_high_rank_many_rows(dev, M, K, R, fp4, smooth):
     not fill the last rank tile pair (96, 112), NVFP4, no smoothing, K beyond what LDS holds of smoothing factors.  The
     oracle runs on a sample of the rows (they are independent), all padding rows are checked to be zero."""
     announce(f"quantize high rank M={M} K={K} R={R} fp4={fp4} smooth={smooth}")
+    _check_row_sample(dev, M, K, R, fp4, smooth)
+
+
+@pytest.mark.parametrize("M,K,R,fp4", [(4608, 256, 32, False), (9000, 384, 32, False), (4500, 6272, 16, False), (2300, 256, 128, False),
+                                       (2300, 384, 64, False), (9000, 256, 128, False), (2300, 256, 256, False), (1000, 256, 144, False),
+                                       (4608, 256, 32, True), (2300, 256, 128, True), (2300, 384, 64, True), (9000, 256, 32, True)])
+def test_workgroup_shapes_by_rows_and_rank(dev, M, K, R, fp4):
+    """The launcher picks the workgroup's shape (waves, rows, requests ahead, rows or chunks split among the waves) by
+    precision, rank, row count and row length; one case per branch of that choice beyond those the other tests take:
+    32 rows on eight waves (M = 4608; long rows; ranks 64 and 128 from 8 rows per compute unit on; the windows of rank
+    256), 16 rows on four waves with two chunks ahead (many short rows; NVFP4 at 4608 rows and at rank 128; few rows at
+    ranks above 128), the rows-split form from 32 rows per compute unit on at rank 128."""
+    announce(f"quantize workgroup shapes M={M} K={K} R={R} fp4={fp4}")
+    _check_row_sample(dev, M, K, R, fp4, True)
+
+
+def _check_row_sample(dev, M, K, R, fp4, smooth):
     layer = synth.make_layer(128, K, R, seed=R + K, fp4=fp4)
     x = synth.make_activations(M, K, seed=M % 1000 + K)
     codes, osc, la = _run(dev, x, layer, fp4=fp4, smooth=smooth)
