@@ -372,21 +372,21 @@ int gemm_fp4(const svdq_gemm_args *a, hipStream_t st, int dev, int ncu, bool noa
         // travel through the workspace (M = 4608, N = 21504: 252 workgroups x 6 tiles 549 us, 256 even shares 560).
         nwg = divisor;
     } else if (ntiles < ncu) {
-        // Fewer tiles than compute units.  A workgroup alone on its compute unit takes 1.67 us per k-group; the parties
-        // of a tile meet through the workspace, which costs the last one about 12 us + 20 us per party beyond itself
-        // (measured: 12 tiles at K = 3072, whole 80 us, two parties 72; at K = 12288 whole 290, eight parties 183; 144
-        // tiles at K = 3072 whole 85, split over all compute units 109).  So: whole tiles unless a split into equal
+        // Fewer tiles than compute units.  A workgroup alone on its compute unit takes 1.3 us per k-group plus 12 us; the
+        // parties of a tile meet through the workspace, which costs about 6 us + 13.5 us per party (measured, 12 tiles:
+        // K = 3072 whole 74.6 us, two / three / four parties 63.0 / 64.0 / 69.8; K = 12288 whole 256.8, two / three /
+        // four / six / eight parties 158.1 / 130.2 / 122.4 / 126.2 / 139.0).  So: whole tiles unless a split into equal
         // parts pays by that count, or the caller asks for k_split parts.
         const int kg = (int)(a->K / 64);
         int parties = 1;
         if (a->k_split > 1) {
             parties = (int)a->k_split;
         } else {
-            double best = 1.67 * kg;
+            double best = 1.3 * kg + 12.0;
             for (int cand : {2, 3, 4, 6, 8}) {
                 if (ntiles * cand > ncu || kg / cand < 12) break;
-                const double t = 1.67 * kg / cand + 12.0 + 20.0 * (cand - 1);
-                if (t < 0.9 * best) {
+                const double t = 1.3 * kg / cand + 6.0 + 13.5 * cand;
+                if (t < (parties == 1 ? 0.90 : 0.95) * best) {  // a split has to pay clearly; more parts likewise
                     best = t;
                     parties = cand;
                 }
