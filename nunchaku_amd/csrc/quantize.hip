@@ -413,7 +413,8 @@ int dispatch(const QuantParams &p, hipStream_t stream) {
         // Up to one 16-row workgroup per compute unit (256 of them) the walk over K is what takes the time: eight waves
         // split it (M = 256 ... 4096 at K = 3072: 7.9 ... 10.1 us against 9.0 ... 11.3 with four; K = 12288, M = 256:
         // 19.6 against 25.5).
-        if (RT <= 2 && p.M_pad <= 16 * ncu) return launch<8, 1, 2, 1, FP4, false>(p, stream);
+        // (two chunks requested ahead: the same at K = 3072, M = 256 and K = 12288: 16.5 us against 20.1)
+        if (RT <= 2 && p.M_pad <= 16 * ncu) return launch<8, 1, 2, 2, FP4, false>(p, stream);
         // Beyond that, at ranks up to 32 (measured at K = 3072 unless noted, on 256 compute units):
         //   up to two 16-row blocks per compute unit, and long rows at any M: eight waves on 32 rows, fewer workgroups
         //   than compute units included (M = 4608: 11.5 us against 12.6 for one workgroup per compute unit with equal
