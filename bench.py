@@ -49,8 +49,8 @@ PROFILED_GEMM_FETCH_WRITE_KIB = {
     "flux_mlp_fc2": (154337.3, 27648.0),
     "qwen_batched_r128": (696300.5, 442369.8),
     "c1_small": (12820.6, 10755.0),
-    "flux_single_nvfp4": (151611.5, 215470.7),
-    "flux_single_out_nvfp4": (122092.9, 31320.1),
+    "flux_single_nvfp4": (146101.8, 197586.7),
+    "flux_single_out_nvfp4": (121730.6, 28944.1),
 }
 PROFILED_GEMM_TRAFFIC_BYTES = {w: (FETCH_SCALE * f + WRITE_SCALE * wr) * 1024 for w, (f, wr) in PROFILED_GEMM_FETCH_WRITE_KIB.items()}
 HBM_PEAK_GBS = 8000.0

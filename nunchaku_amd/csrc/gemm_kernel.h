@@ -169,7 +169,7 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     struct TileCtx {
         int tile, gb, ge;  // k-groups [gb, ge) of the tile
         int m0, n0, shift;
-        bool col_ok;
+        int col_ok;
         const uint8_t *a_ptr, *b_ptr, *as_ptr, *bs_ptr;
     };
     // follow: the segment after the one given by prev_* (the next tile, from its first k-group), without divisions
@@ -428,8 +428,6 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
     const int wm = wave >> 1, wn = wave & 1, r32 = lane & 31, h = lane >> 5;
     const int m0 = cur.m0, n0 = cur.n0, tile_e = cur.tile;
     const int *tile_shift = rowshift + ti * 256;
-    TileCtx nxt = cur;
-    if (have_next) nxt = make_ctx(batch0 + ti + 1, ti + 1, tid, true, cur.tile, cur.m0, cur.n0);
 
     // ---- a tile shared with other workgroups ---------------------------------------------------
     // Every party holds the sum over its part of K.  Whoever finishes last adds all parties' sums in ascending order
@@ -835,7 +833,9 @@ __global__ void __launch_bounds__(256, 1) gemm_w4a4_kernel(GemmParams p) {
         slab_epilogue(std::integral_constant<int, 2>{}, std::true_type{});
         slab_epilogue(std::integral_constant<int, 3>{}, std::true_type{});
     }
-    if (have_next) cur = nxt;
+    // (the next tile's context is worked out here, behind the epilogue: its four addresses would otherwise sit in
+    // scratch memory while the epilogue needs the registers)
+    if (have_next) cur = make_ctx(batch0 + ti + 1, ti + 1, threadIdx.x, true, tile_e, m0, n0);
     __syncthreads();
    }  // tiles of the batch
   }    // batches
